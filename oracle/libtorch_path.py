@@ -1,0 +1,82 @@
+"""The reference's LibTorch path, restated call for call -- TEST INFRASTRUCTURE.
+
+The reference computes its parity targets by handing tensors to LibTorch (a
+third-party dependency pinned at 2.9.1 in the reference's Readme.md:37; the
+``torch`` package importable here is 2.10).  Its FFI adds nothing but
+refcounting around these calls, so the restatement is the calls themselves:
+
+* ``sdpa_4d``       cc/src/tyr.cpp:2563-2589  torch::scaled_dot_product_attention(q,k,v,nullopt,p,is_causal)
+* ``sdpa_gqa_qkv``  cc/src/tyr.cpp:4100-4133  repeat_interleave(n_head/n_kv_head, dim=1) on K and V, then the same call
+* ``mm``            cc/src/tyr.cpp:1602-1607  torch::mm
+* ``fp8_mm``        no LibTorch fp8 GEMM exists in the reference; the parity target for the DSL kernel
+                    (Tyr/GPU/Kernels/PrecisionGemm.lean:97-115) is dequantise -> f32 torch::mm -> scale
+* ``reference_attention`` Examples/GPU/RunFlashAttn.lean:26-48: bf16-rounded inputs, f32 math, O and LSE
+* ``make_inputs``   cc/src/tyr.cpp:424-432,545-551,4246-4250: manual_seed, randn, .to(bfloat16)
+
+Everything here runs on CPU tensors.  It is used as a checker and as the timed
+CPU baseline; the product never imports it.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def make_inputs(seed: int, *shapes, dtype=torch.bfloat16, std: float = 1.0):
+    """manual_seed(seed) then one randn per shape, in order, each cast to ``dtype``."""
+    torch.manual_seed(seed)
+    out = []
+    for s in shapes:
+        t = torch.randn(*s, dtype=torch.float32)
+        if std != 1.0:
+            t = t * std
+        out.append(t.to(dtype))
+    return out
+
+
+def sdpa_4d(q, k, v, is_causal: bool, dropout_p: float = 0.0):
+    return F.scaled_dot_product_attention(q, k, v, None, dropout_p, is_causal)
+
+
+def sdpa_gqa_qkv(q, k, v, is_causal: bool = False, enable_gqa: bool = True, dropout_p: float = 0.0):
+    n_head, n_kv_head = q.shape[1], k.shape[1]
+    if enable_gqa and n_head != n_kv_head and n_kv_head > 0:
+        rep = n_head // n_kv_head
+        k = k.repeat_interleave(rep, 1)
+        v = v.repeat_interleave(rep, 1)
+    return F.scaled_dot_product_attention(q, k, v, None, dropout_p, is_causal)
+
+
+def mm(a, b):
+    return torch.mm(a, b)
+
+
+def fp8_mm(aq, bq, scale_a: float, scale_b: float):
+    """aq [M,K], bq [K,N] float8_e4m3fn -> f32 (scale_a*scale_b) * (deq(aq) @ deq(bq))."""
+    return torch.mm(aq.to(torch.float32), bq.to(torch.float32)) * (float(scale_a) * float(scale_b))
+
+
+def quantize_e4m3(x: torch.Tensor):
+    """Per-tensor absmax quantisation: s = absmax/448, xq = e4m3fn(x/s).  -> (xq, s)"""
+    s = float(x.abs().max()) / 448.0
+    if s == 0.0:
+        s = 1.0
+    xq = (x.to(torch.float32) / s).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return xq, s
+
+
+def reference_attention(q, k, v, is_causal: bool, scale: float | None = None):
+    """f32 attention from the (already rounded) inputs, with LSE = ln sum exp(scaled scores)."""
+    q32, k32, v32 = q.float(), k.float(), v.float()
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    s = torch.matmul(q32, k32.transpose(-1, -2)) * scale
+    if is_causal:
+        n, m = s.shape[-2], s.shape[-1]
+        mask = torch.ones(n, m, dtype=torch.bool).tril(diagonal=m - n)
+        s = s.masked_fill(~mask, float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)
+    o = torch.matmul(torch.softmax(s, dim=-1), v32)
+    return o, lse
