@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-extra]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  The headline workload is the causal flash-attention forward the target is quoted on
+(bf16, B=16 H=16 N=4096 D=128); the other three configurations (GQA decode, bf16 GEMM, fp8 GEMM)
+are measured in the same run and reported under "other_workloads" of the single JSON line.
+
+FLOP / byte conventions (algorithmic work, fixed per configuration):
+  attn_fwd_causal : 4*B*H*N^2*D / 2 FLOP (two GEMMs, causal half)           -> MFMA bf16 2.5 PFLOP/s
+  gqa_decode      : bytes of K + V + Q + O                                   -> HBM 8 TB/s
+  gemm_bf16       : 2*M*N*K FLOP                                             -> MFMA bf16 2.5 PFLOP/s
+  gemm_fp8        : 2*M*N*K FLOP                                             -> MFMA fp8 5.0 PFLOP/s
+Kernel durations are measured with HIP events on the stream the kernels are launched on.
+The CPU baseline runs the reference's LibTorch call sequence (oracle/libtorch_path.py) on the host
+cores of this box over a bounded sample of the same workload; it is a reported baseline only.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK = {"mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "hbm": 8000.0}   # TFLOP/s, TFLOP/s, GB/s
+
+
+def _events(torch, n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_steps(torch, fn, steps, warmup):
+    """Runs warmup + steps launches of fn on the current stream; returns (wall ms/step, event ms/step)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = _events(torch, 2)
+    t0 = time.perf_counter()
+    ev[0].record()
+    for _ in range(steps):
+        fn()
+    ev[1].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, ev[0].elapsed_time(ev[1]) / steps
+
+
+# ------------------------------------------------------------------------------- workloads
+
+def wl_attn(torch, tyr, steps, warmup, cpu):
+    B, H, N, D = 16, 16, 4096, 128
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(3))
+    sc = 1.0 / math.sqrt(D)
+    fn = lambda: tyr.flash_attn_fwd(q, k, v, causal=True, scale=sc)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    flop = 4.0 * B * H * N * N * D / 2.0
+    tf = flop / (ms * 1e-3) / 1e12
+    res = {
+        "metric": "attn fwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+        "dtype": "bf16",
+        "config": {"workload": "causal flash-attention forward, bf16, B=16 H=16 N=4096 D=128, O + LSE",
+                   "flop_convention": "4*B*H*N^2*D/2 (causal half)", "scale": "1/sqrt(128)"},
+        "roofline": {"bound": "mfma", "kernel": "flash_attn_fwd_kernel<128,true>", "achieved": tf,
+                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"], "traffic": None},
+    }
+    if cpu:
+        from oracle import libtorch_path as lt
+        hs = 16                                    # sample: one batch entry (16 of the 256 heads)
+        qc, kc, vc = (t[:1, :hs].cpu() for t in (q, k, v))
+        lt.sdpa_4d(qc[:, :2], kc[:, :2], vc[:, :2], True)   # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 50):
+            lt.sdpa_4d(qc, kc, vc, True)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": (4.0 * hs * N * N * D / 2.0) / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU scaled_dot_product_attention(is_causal) on 1 of 16 batch "
+                                         f"entries (16 heads, N=4096, D=128, bf16), {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_decode(torch, tyr, steps, warmup, cpu):
+    B, Hq, Hkv, L, D = 32, 32, 8, 8192, 128
+    torch.manual_seed(1)
+    q = torch.randn(B, Hq, 1, D, device="cuda").to(torch.bfloat16)
+    # rotate over 4 independent caches (1.07 GB each) so no launch finds its K/V in the 256 MB last-level cache
+    caches = [(torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16),
+               torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16)) for _ in range(4)]
+    sc = 1.0 / math.sqrt(D)
+    it = [0]
+
+    def fn():
+        k, v = caches[it[0] % len(caches)]
+        it[0] += 1
+        return tyr.gqa_decode(q, k, v, scale=sc)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    nbytes = 2 * B * Hkv * L * D * 2 + 2 * B * Hq * D * 2
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    res = {
+        "metric": "decode attn GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+        "dtype": "bf16",
+        "config": {"workload": "GQA decode attention, bf16, batch 32, 32 q heads, 8 kv heads, D=128, KV length 8192",
+                   "bytes_convention": "K + V + Q + O = 1,074,266,112 B (split partials excluded)",
+                   "num_splits": int(__import__("tyr_amd._lib", fromlist=["load"]).load()
+                                     .tyr_hip_gqa_decode_auto_splits(B, Hkv, L)),
+                   "note": "time covers both passes (split kernel + combine kernel)"},
+        "roofline": {"bound": "hbm", "kernel": "gqa_decode_split_kernel (+combine)", "achieved": gbs,
+                     "peak": PEAK["hbm"], "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": None},
+    }
+    if cpu:
+        from oracle import libtorch_path as lt
+        nb = 4                                     # sample: 4 of the 32 sequences
+        qc = q[:nb].cpu()
+        kc, vc = (t[:nb].cpu() for t in caches[0])
+        lt.sdpa_gqa_qkv(qc[:1], kc[:1], vc[:1])
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 8 and reps < 50):
+            lt.sdpa_gqa_qkv(qc, kc, vc)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": nbytes * nb / B / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"LibTorch CPU repeat_interleave + scaled_dot_product_attention on {nb} of 32 "
+                                         f"sequences, {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_gemm_bf16(torch, tyr, steps, warmup, cpu):
+    M = N = K = 4096
+    torch.manual_seed(2)
+    a = (torch.randn(M, K, device="cuda") * K ** -0.25).to(torch.bfloat16)
+    b = (torch.randn(K, N, device="cuda") * K ** -0.25).to(torch.bfloat16)
+    fn = lambda: tyr.gemm_bf16(a, b)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+    res = {
+        "metric": "GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+        "dtype": "bf16",
+        "config": {"workload": "bf16 GEMM M=N=K=4096, row-major A and B, f32 accumulate, bf16 out",
+                   "input_std": "K^-1/4 = 0.125"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel<false,false>", "achieved": tf,
+                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"], "traffic": None},
+    }
+    if cpu:
+        from oracle import libtorch_path as lt
+        ac, bc = a.cpu(), b.cpu()
+        lt.mm(ac[:256], bc)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 8 and reps < 50):
+            lt.mm(ac, bc)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"LibTorch CPU torch.mm (bf16) on the full 4096^3 problem, "
+                                                         f"{reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_gemm_fp8(torch, tyr, steps, warmup, cpu):
+    M = N = K = 8192
+    torch.manual_seed(3)
+    aq, sa = tyr.quantize_e4m3(torch.randn(M, K, device="cuda"))
+    bq, sb = tyr.quantize_e4m3(torch.randn(K, N, device="cuda"))
+    fn = lambda: tyr.gemm_fp8(aq, bq, sa, sb)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+    res = {
+        "metric": "GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+        "dtype": "fp8_e4m3",
+        "config": {"workload": "fp8 e4m3 GEMM M=N=K=8192, per-tensor f32 scales, bf16 out"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_fp8_kernel<false,false>", "achieved": tf,
+                     "peak": PEAK["mfma_fp8"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_fp8"], "traffic": None},
+    }
+    if cpu:
+        from oracle import libtorch_path as lt
+        rows = 1024                                # sample: 1/8 of the rows of A
+        ac, bc = aq[:rows].cpu(), bq.cpu()
+        lt.fp8_mm(ac[:64], bc, sa, sb)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or (time.perf_counter() - t0 < 8 and reps < 20):
+            lt.fp8_mm(ac, bc, sa, sb)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU dequantise + f32 torch.mm on {rows} of 8192 rows of A, "
+                                         f"{reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+WORKLOADS = {"attn_fwd_causal": wl_attn, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16, "gemm_fp8": wl_gemm_fp8}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="attn_fwd_causal", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
+        return 2
+
+    import torch
+    import tyr_amd
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False).", file=sys.stderr)
+        return 3
+    torch.cuda.set_device(0)
+    info = tyr_amd.device_info(0)
+
+    head = WORKLOADS[args.workload](torch, tyr_amd, args.steps, args.warmup, not args.no_cpu)
+    line = {
+        "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
+        "cpu_baseline": head.get("cpu_baseline"), "wall_ms_per_step": round(head["wall_ms_per_step"], 5),
+        "device": info,
+    }
+    if not args.no_extra:
+        others = []
+        for name, fn in WORKLOADS.items():
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            r = fn(torch, tyr_amd, max(10, args.steps // 2), max(3, args.warmup // 2), not args.no_cpu)
+            r["workload"] = name
+            others.append(r)
+        line["other_workloads"] = others
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

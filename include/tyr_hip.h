@@ -1,0 +1,140 @@
+/*
+ * tyr_hip.h -- C ABI of the gfx950 (MI355X) kernel library behind Tyr's GPU surface.
+ *
+ * Plain pointers and sizes only: no torch, no Lean types.  Every pointer is a
+ * device pointer into HBM unless stated otherwise; every tensor is dense and
+ * row-major ("contiguous") with the stated shape.  `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  Launches are asynchronous on
+ * that stream; the caller synchronises, exactly as with the reference's
+ * generated launchers (Tyr/GPU/Codegen/Attribute.lean:346-386: launch, then
+ * cudaGetLastError, no synchronisation).
+ *
+ * All functions return TYR_HIP_OK (0) or a negative tyr_hip_status; they never
+ * throw and never abort.  tyr_hip_strerror() gives the message a Lean wrapper
+ * puts into `IO.userError` (the reference's convention,
+ * Tyr/GPU/Codegen/Attribute.lean:334-336,380-384).
+ *
+ * bf16 tensors are uint16 bit patterns in memory; e4m3 tensors are OCP FP8
+ * E4M3 ("e4m3fn": bias 7, max 448, no infinity) bytes.
+ */
+#ifndef TYR_HIP_H
+#define TYR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tyr_hip_status {
+    TYR_HIP_OK = 0,
+    TYR_HIP_ERR_NULL_POINTER = -1,   /* a required pointer argument is NULL            */
+    TYR_HIP_ERR_BAD_SHAPE = -2,      /* zero/negative/inconsistent extents             */
+    TYR_HIP_ERR_UNSUPPORTED = -3,    /* valid request the kernels do not implement     */
+    TYR_HIP_ERR_MISALIGNED = -4,     /* pointer or row pitch not 16-byte aligned       */
+    TYR_HIP_ERR_WORKSPACE = -5,      /* workspace missing or too small                 */
+    TYR_HIP_ERR_LAUNCH = -6,         /* HIP reported a launch error                    */
+    TYR_HIP_ERR_NO_DEVICE = -7,      /* no gfx950 device / library built without HIP   */
+    TYR_HIP_ERR_NOT_DEVICE_MEMORY = -8 /* tyr_hip_check_device_pointer: host pointer   */
+} tyr_hip_status;
+
+/* Message for a status code; static storage, never NULL. */
+const char* tyr_hip_strerror(int status);
+
+/* Library/ABI version (major*10000 + minor*100 + patch). */
+int tyr_hip_version(void);
+
+/* Fills the properties the harness prints next to every figure.  Any pointer may be NULL.
+ * Returns TYR_HIP_ERR_NO_DEVICE when no GPU is visible. */
+int tyr_hip_device_info(int device, char* name, size_t name_len, int* compute_units,
+                        int* lds_bytes_per_cu, int* clock_mhz, size_t* hbm_bytes);
+
+/* The "<p> must be a CUDA tensor" check of the reference's launcher
+ * (Tyr/GPU/Codegen/Attribute.lean:334), for callers that hold raw pointers:
+ * TYR_HIP_OK if `p` is device memory, TYR_HIP_ERR_NOT_DEVICE_MEMORY otherwise. */
+int tyr_hip_check_device_pointer(const void* p);
+
+/* ---------------------------------------------------------------------------
+ * Flash-attention forward:  O = softmax(Q K^T * scale [+ causal mask]) V,
+ * LSE[b,h,i] = ln sum_j exp(scale * q_i . k_j)   (natural log of the scaled scores).
+ *
+ * Replaces the reference's DSL attention forward kernels and their launchers
+ * (Tyr/GPU/Kernels/MhaH100.lean:71-128 `tkFlashAttnFwd2BlockLse`,
+ *  Tyr/GPU/Kernels/MhaH100LCF.lean:29-132 for D=128; launcher text
+ *  Tyr/GPU/Codegen/Attribute.lean:346-386) and is the GPU twin of
+ * `lean_torch_sdpa_4d` (cc/src/tyr.cpp:2563-2589).
+ *
+ *   q, k, v : bf16 [B, H, N, D]        o : bf16 [B, H, N, D]
+ *   lse     : f32  [B, H, N]  (may be NULL: not written)
+ *   causal  : 0/1, key j visible to query i iff j <= i
+ *   scale   : multiplies Q K^T (pass 1/sqrt(D) for the usual attention)
+ * Supported: D in {64, 128}; any N >= 1; B*H*ceil(N/128) < 2^31.
+ */
+int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                           uint64_t B, uint64_t H, uint64_t N, uint64_t D,
+                           int causal, float scale, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * GQA decode attention (one query token per sequence), split-KV + LSE combine.
+ *
+ * GPU twin of `lean_torch_sdpa_gqa_qkv` with q_seq = 1, is_causal = false,
+ * enable_gqa = true (cc/src/tyr.cpp:4100-4133; caller
+ * Tyr/Model/Qwen/Attention.lean:151-211); query head h reads kv head
+ * h / (Hq/Hkv) (repeat_interleave along the head axis).  The packing of the
+ * Hq/Hkv query heads of one kv head into one MFMA tile follows
+ * Tyr/GPU/Kernels/FlashAttn3.lean:535-624.
+ *
+ *   q : bf16 [B, Hq, 1, D]
+ *   k, v : bf16 [B, Hkv, kv_stride, D]; only rows [0, L) of each (b, kv head) are read.
+ *          kv_stride >= L is the allocated cache length (the reference's
+ *          [batch, kv_heads, maxLen, head_dim] cache, Tyr/Model/Qwen/Attention.lean:54-68).
+ *   o : bf16 [B, Hq, 1, D]      lse : f32 [B, Hq] (may be NULL)
+ *   num_splits : KV chunks per (b, kv head); 0 = choose automatically.
+ *   workspace  : device scratch of at least tyr_hip_gqa_decode_workspace_bytes(...) bytes,
+ *                16-byte aligned; contents need not be initialised.
+ * Supported: D == 128; 1 <= Hq/Hkv <= 16 with Hq % Hkv == 0; L >= 1; num_splits <= 64.
+ */
+size_t tyr_hip_gqa_decode_workspace_bytes(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L,
+                                          uint64_t D, uint64_t num_splits);
+/* The split count the library uses when num_splits == 0 is passed. */
+uint64_t tyr_hip_gqa_decode_auto_splits(uint64_t B, uint64_t Hkv, uint64_t L);
+int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse,
+                       uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                       uint64_t kv_stride, float scale, uint64_t num_splits,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * bf16 GEMM, f32 accumulation, bf16 output:  C = A B  (trans_b = 0, B is [K, N])
+ *                                            C = A B^T (trans_b = 1, B is [N, K]).
+ *
+ * Replaces `tkH100Bf16GemmFwd` (Tyr/GPU/Kernels/Bf16Gemm.lean:64-73) over
+ * `tiledAccumulator` (Tyr/GPU/Kernels/GemmCommon.lean:22-69, the N x K form)
+ * and `simpleGemm` (Tyr/GPU/Kernels/Examples.lean:23-65, the K x N form);
+ * GPU twin of `lean_torch_mm` (cc/src/tyr.cpp:1602-1607).
+ *
+ *   a : bf16 [M, K]   b : bf16 [K, N] or [N, K]   c : bf16 [M, N]
+ * Supported: M, N, K >= 1 with K % 8 == 0 and N % 8 == 0 (16-byte rows).
+ */
+int tyr_hip_gemm_bf16(const void* a, const void* b, void* c,
+                      uint64_t M, uint64_t N, uint64_t K, int trans_b, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * FP8 E4M3 GEMM with per-tensor f32 scales, bf16 output:
+ *     C = bf16( scale_a * scale_b * (Aq Bq) ),  f32 accumulation, scale in the epilogue.
+ *
+ * Replaces `gemmFp8E4M3Fwd` / `tkH100Fp8ScaledGemmFwd`
+ * (Tyr/GPU/Kernels/PrecisionGemm.lean:97-115,178-189) with the scalar epilogue of
+ * `applyGlobalScalar` (Tyr/GPU/Kernels/GemmCommon.lean:135-144).
+ *
+ *   aq : e4m3 [M, K]   bq : e4m3 [K, N] (trans_b = 0) or [N, K] (trans_b = 1)   c : bf16 [M, N]
+ * Supported: M, N, K >= 1 with K % 16 == 0 and N % 16 == 0 (16-byte rows).
+ */
+int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c,
+                     uint64_t M, uint64_t N, uint64_t K,
+                     float scale_a, float scale_b, int trans_b, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TYR_HIP_H */

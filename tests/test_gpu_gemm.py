@@ -1,0 +1,134 @@
+"""Parity of the gfx950 GEMM kernels (through the C ABI) with the CPU checker.
+
+Tolerance (stated by the task): relative Frobenius error <= 1e-2 against an fp32 reference of
+the rounded operands.  Small cases are also held to one bf16 ulp of the row magnitude against
+the scalar C restatement, and structured operands (identity, permutation) must be bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import libtorch_path as lt
+from tests.util import bits, from_bits, rel_fro, u8
+
+pytestmark = pytest.mark.gpu
+TOL_FRO = 1e-2
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import tyr_amd
+    return tyr_amd
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 512, 4096), (8, 8, 8),
+                                   (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256)])
+def test_gemm_bf16_matches_oracle(gpu, M, N, K, trans_b):
+    a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
+    bb = b.t().contiguous() if trans_b else b
+    c = gpu.gemm_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
+    want_bits = oracle.gemm_bf16(bits(a), bits(bb), trans_b=trans_b)
+    want = from_bits(want_bits).float()
+    f32 = a.float() @ b.float()
+    assert rel_fro(c, f32) <= TOL_FRO
+    # accumulation order differs, so allow one bf16 ulp of the largest magnitude in the result
+    assert float((c.float() - want).abs().max()) <= float(want.abs().max()) * 2 ** -7 + 1e-6
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gemm_bf16_identity_and_permutation_bit_exact(gpu, trans_b):
+    n = 512
+    a, = lt.make_inputs(7, (n, n))
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(0))
+    P = torch.eye(n)[perm].to(torch.bfloat16)
+    Pb = P.t().contiguous() if trans_b else P
+    ab = a.t().contiguous() if trans_b else a
+    got_pa = gpu.gemm_bf16(P.cuda(), ab.cuda(), trans_b=trans_b).cpu()      # rows of A permuted
+    got_ap = gpu.gemm_bf16(a.cuda(), Pb.cuda(), trans_b=trans_b).cpu()      # columns of A permuted
+    assert np.array_equal(bits(got_pa), bits(a[perm]))
+    assert np.array_equal(bits(got_ap), bits(a[:, torch.argsort(perm)]))
+
+
+def test_gemm_bf16_full_size_config(gpu):
+    # M = N = K = 4096, entries ~ N(0, 1/sqrt(K)) (std K^-1/4), row-major A and B.
+    M = N = K = 4096
+    a, b = lt.make_inputs(2, (M, K), (K, N), std=K ** -0.25)
+    a, b = a.cuda(), b.cuda()
+    c = gpu.gemm_bf16(a, b)
+    ref = a.float() @ b.float()                      # fp32 reference of the bf16-rounded inputs
+    assert rel_fro(c, ref) <= TOL_FRO
+    # a 64-row slab against the scalar C restatement
+    rows = slice(1000, 1064)
+    want = from_bits(oracle.gemm_bf16(bits(a[rows]), bits(b))).float()
+    assert float((c[rows].cpu().float() - want).abs().max()) <= float(want.abs().max()) * 2 ** -7
+    # linearity in a power of two is exact
+    c2 = gpu.gemm_bf16((a.float() * 2).to(torch.bfloat16), b)
+    assert torch.equal(c2.float(), c.float() * 2)
+    # NT on the transposed operand gives the same bits as NN (same k order per output)
+    cnt = gpu.gemm_bf16(a, b.t().contiguous(), trans_b=True)
+    assert rel_fro(cnt, ref) <= TOL_FRO
+    # determinism
+    assert torch.equal(gpu.gemm_bf16(a, b), c)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 256, 384), (16, 16, 16), (300, 272, 80),
+                                   (1, 16, 16), (257, 48, 1040)])
+def test_gemm_fp8_matches_oracle(gpu, M, N, K, trans_b):
+    torch.manual_seed(200 + M + N + K)
+    a, b = torch.randn(M, K), torch.randn(K, N)
+    aq, sa = lt.quantize_e4m3(a)
+    bq, sb = lt.quantize_e4m3(b)
+    bqb = bq.t().contiguous() if trans_b else bq
+    c = gpu.gemm_fp8(aq.cuda(), bqb.cuda(), sa, sb, trans_b=trans_b).cpu()
+    want_bits, want_f32 = oracle.gemm_fp8(u8(aq), u8(bqb), sa, sb, trans_b=trans_b)
+    ref = lt.fp8_mm(aq, bq, sa, sb)                  # fp32 GEMM of the dequantised operands
+    assert rel_fro(c, ref) <= TOL_FRO
+    # products of e4m3 values are exact in f32; only the summation order differs
+    assert float((c.float() - torch.from_numpy(want_f32)).abs().max()) <= float(ref.abs().max()) * 2 ** -7 + 1e-6
+
+
+def test_gemm_fp8_every_code_decodes_like_ocp_e4m3(gpu):
+    # B = identity (1.0 = 0x38): C = decode(Aq) * sa * sb exactly (every product is exact, one term per sum)
+    tab = oracle.e4m3_table()
+    codes = np.array([c for c in range(256) if not np.isnan(tab[c])], dtype=np.uint8)
+    A = np.zeros((256, 256), np.uint8)
+    A.flat[:codes.size] = codes
+    eye = np.zeros((256, 256), np.uint8)
+    np.fill_diagonal(eye, 0x38)
+    aq = torch.from_numpy(A).view(torch.float8_e4m3fn).cuda()
+    for trans_b in (False, True):
+        c = gpu.gemm_fp8(aq, torch.from_numpy(eye).view(torch.float8_e4m3fn).cuda(), 0.5, 4.0, trans_b=trans_b).cpu()
+        want = torch.from_numpy(tab[A] * 2.0).to(torch.bfloat16)     # e4m3 values are exact in bf16
+        assert np.array_equal(bits(c), bits(want))
+
+
+def test_gemm_fp8_full_size_config(gpu):
+    # M = N = K = 8192, values ~ N(0,1) quantised with absmax scaling.
+    M = N = K = 8192
+    torch.manual_seed(5)
+    a = torch.randn(M, K, device="cuda")
+    b = torch.randn(K, N, device="cuda")
+    from tyr_amd import quantize_e4m3
+    aq, sa = quantize_e4m3(a)
+    bq, sb = quantize_e4m3(b)
+    c = gpu.gemm_fp8(aq, bq, sa, sb)
+    ref = (aq.float() @ bq.float()) * (sa * sb)      # fp32 GEMM of the dequantised operands (GPU, checker only)
+    assert rel_fro(c, ref) <= TOL_FRO
+    rows = slice(4000, 4016)
+    _, want = oracle.gemm_fp8(u8(aq[rows]), u8(bq), sa, sb)
+    assert float((c[rows].cpu().float() - torch.from_numpy(want)).abs().max()) <= float(np.abs(want).max()) * 2 ** -7
+    assert torch.equal(gpu.gemm_fp8(aq, bq, sa, sb), c)
+
+
+def test_error_convention(gpu):
+    from tyr_amd import TyrGpuError
+    a = torch.zeros(16, 16, dtype=torch.bfloat16)
+    with pytest.raises(TyrGpuError, match="a must be a CUDA tensor"):
+        gpu.gemm_bf16(a, a.cuda())
+    with pytest.raises(TyrGpuError, match="b must be contiguous"):
+        gpu.gemm_bf16(a.cuda(), torch.zeros(32, 16, dtype=torch.bfloat16).cuda()[::2])
+    with pytest.raises(TyrGpuError, match="not supported"):
+        gpu.gemm_bf16(torch.zeros(16, 12, dtype=torch.bfloat16).cuda(), torch.zeros(12, 16, dtype=torch.bfloat16).cuda())

@@ -1,0 +1,53 @@
+"""ctypes binding of libtyr_hip.so.  There is no fallback: a missing library is an error."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtyr_hip.so")
+
+# every symbol include/tyr_hip.h declares
+SYMBOLS = (
+    "tyr_hip_strerror", "tyr_hip_version", "tyr_hip_device_info", "tyr_hip_check_device_pointer",
+    "tyr_hip_flash_attn_fwd", "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
+    "tyr_hip_gqa_decode", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
+)
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C tyr_amd/csrc` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`). "
+            "tyr_amd has no CPU or PyTorch fallback.")
+    L = ctypes.CDLL(LIB_PATH)
+    u64, vp, ci, f32, sz = ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+    L.tyr_hip_strerror.argtypes = [ci]
+    L.tyr_hip_strerror.restype = ctypes.c_char_p
+    L.tyr_hip_version.argtypes = []
+    L.tyr_hip_version.restype = ci
+    L.tyr_hip_device_info.argtypes = [ci, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
+                                      ctypes.POINTER(ci), ctypes.POINTER(sz)]
+    L.tyr_hip_device_info.restype = ci
+    L.tyr_hip_check_device_pointer.argtypes = [vp]
+    L.tyr_hip_check_device_pointer.restype = ci
+    L.tyr_hip_flash_attn_fwd.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, ci, f32, vp]
+    L.tyr_hip_flash_attn_fwd.restype = ci
+    L.tyr_hip_gqa_decode_workspace_bytes.argtypes = [u64] * 6
+    L.tyr_hip_gqa_decode_workspace_bytes.restype = sz
+    L.tyr_hip_gqa_decode_auto_splits.argtypes = [u64] * 3
+    L.tyr_hip_gqa_decode_auto_splits.restype = u64
+    L.tyr_hip_gqa_decode.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, u64, u64, f32, u64, vp, sz, vp]
+    L.tyr_hip_gqa_decode.restype = ci
+    L.tyr_hip_gemm_bf16.argtypes = [vp, vp, vp, u64, u64, u64, ci, vp]
+    L.tyr_hip_gemm_bf16.restype = ci
+    L.tyr_hip_gemm_fp8.argtypes = [vp, vp, vp, u64, u64, u64, f32, f32, ci, vp]
+    L.tyr_hip_gemm_fp8.restype = ci
+    _lib = L
+    return L

@@ -1,0 +1,160 @@
+// C ABI of the library (declared in include/tyr_hip.h): argument validation and dispatch.
+// Validation mirrors what the reference's generated launchers check before a launch
+// (Tyr/GPU/Codegen/Attribute.lean:331-386): every failure is reported through the return
+// value, nothing throws, nothing is launched on invalid input.
+#include "../../include/tyr_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <limits.h>
+#include <string.h>
+
+#include "launch.hpp"
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool fits_int(uint64_t v) { return v <= (uint64_t)INT_MAX; }
+
+constexpr uint64_t kMaxSplits = 64;
+
+uint64_t auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {
+    // Aim for about 4 workgroups (16 waves) per CU on 256 CUs with at least 256 kv rows per
+    // workgroup, so that every wave has a few 32-row steps to pipeline.
+    const uint64_t groups = B * Hkv;
+    if (groups == 0) return 1;
+    uint64_t s = (1024 + groups - 1) / groups;
+    const uint64_t max_by_len = L / 256 ? L / 256 : 1;
+    if (s > max_by_len) s = max_by_len;
+    if (s < 1) s = 1;
+    if (s > kMaxSplits) s = kMaxSplits;
+    return s;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* tyr_hip_strerror(int status) {
+    switch (status) {
+        case TYR_HIP_OK: return "ok";
+        case TYR_HIP_ERR_NULL_POINTER: return "a required tensor pointer is null";
+        case TYR_HIP_ERR_BAD_SHAPE: return "tensor extents are zero, too large or inconsistent";
+        case TYR_HIP_ERR_UNSUPPORTED: return "shape or option not supported by the gfx950 kernels";
+        case TYR_HIP_ERR_MISALIGNED: return "tensor pointers and rows must be 16-byte aligned";
+        case TYR_HIP_ERR_WORKSPACE: return "workspace is missing or too small";
+        case TYR_HIP_ERR_LAUNCH: return "HIP reported a kernel launch error";
+        case TYR_HIP_ERR_NO_DEVICE: return "no gfx950 device is available";
+        case TYR_HIP_ERR_NOT_DEVICE_MEMORY: return "pointer must be a CUDA tensor (device memory)";
+        default: return "unknown tyr_hip status";
+    }
+}
+
+int tyr_hip_version(void) { return 100; }
+
+int tyr_hip_device_info(int device, char* name, size_t name_len, int* compute_units,
+                        int* lds_bytes_per_cu, int* clock_mhz, size_t* hbm_bytes) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) {
+        (void)hipGetLastError();
+        return TYR_HIP_ERR_NO_DEVICE;
+    }
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, device) != hipSuccess) return TYR_HIP_ERR_NO_DEVICE;
+    if (name && name_len) {
+        strncpy(name, p.gcnArchName, name_len - 1);
+        name[name_len - 1] = 0;
+    }
+    if (compute_units) *compute_units = p.multiProcessorCount;
+    if (lds_bytes_per_cu) *lds_bytes_per_cu = (int)p.maxSharedMemoryPerMultiProcessor;
+    if (clock_mhz) *clock_mhz = p.clockRate / 1000;
+    if (hbm_bytes) *hbm_bytes = p.totalGlobalMem;
+    return TYR_HIP_OK;
+}
+
+int tyr_hip_check_device_pointer(const void* p) {
+    if (!p) return TYR_HIP_ERR_NULL_POINTER;
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return TYR_HIP_ERR_NOT_DEVICE_MEMORY;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged
+               ? TYR_HIP_OK
+               : TYR_HIP_ERR_NOT_DEVICE_MEMORY;
+}
+
+int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                           uint64_t B, uint64_t H, uint64_t N, uint64_t D, int causal, float scale,
+                           void* stream) {
+    if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
+    if (B == 0 || H == 0 || N == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!fits_int(N) || !fits_int(B * H) || B * H > (uint64_t)INT_MAX / ((N + 127) / 128))
+        return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
+    if (lse && (reinterpret_cast<uintptr_t>(lse) & 3u)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_flash_attn_fwd(q, k, v, o, lse, (int)B, (int)H, (int)N, (int)D,
+                                              causal != 0, scale, static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+uint64_t tyr_hip_gqa_decode_auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {
+    return auto_splits(B, Hkv, L);
+}
+
+size_t tyr_hip_gqa_decode_workspace_bytes(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L,
+                                          uint64_t D, uint64_t num_splits) {
+    if (num_splits == 0) num_splits = auto_splits(B, Hkv, L);
+    return (size_t)(B * Hq * num_splits * (D + 2) * sizeof(float));
+}
+
+int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse,
+                       uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                       uint64_t kv_stride, float scale, uint64_t num_splits, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
+    if (B == 0 || Hq == 0 || Hkv == 0 || L == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (Hq % Hkv != 0 || kv_stride < L) return TYR_HIP_ERR_BAD_SHAPE;
+    if (D != 128 || Hq / Hkv > 16 || num_splits > kMaxSplits) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!fits_int(L) || !fits_int(B * Hq) || B * Hkv > 65535 || kv_stride > (uint64_t)INT_MAX)
+        return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
+    if (num_splits == 0) num_splits = auto_splits(B, Hkv, L);
+    const size_t need = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
+    if (!workspace || workspace_bytes < need) return TYR_HIP_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_gqa_decode(q, k, v, o, lse, (int)B, (int)Hq, (int)Hkv, (int)L, (int)D,
+                                          (int64_t)kv_stride, scale, (int)num_splits, workspace,
+                                          static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_gemm_bf16(const void* a, const void* b, void* c, uint64_t M, uint64_t N, uint64_t K,
+                      int trans_b, void* stream) {
+    if (!a || !b || !c) return TYR_HIP_ERR_NULL_POINTER;
+    if (M == 0 || N == 0 || K == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return TYR_HIP_ERR_BAD_SHAPE;
+    if (((M + 255) / 256) * ((N + 255) / 256) > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
+    if (K % 8 != 0 || N % 8 != 0) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_gemm_bf16(a, b, c, (int)M, (int)N, (int)K, trans_b != 0,
+                                         static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c, uint64_t M, uint64_t N, uint64_t K,
+                     float scale_a, float scale_b, int trans_b, void* stream) {
+    if (!aq || !bq || !c) return TYR_HIP_ERR_NULL_POINTER;
+    if (M == 0 || N == 0 || K == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return TYR_HIP_ERR_BAD_SHAPE;
+    if (((M + 255) / 256) * ((N + 255) / 256) > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
+    if (K % 16 != 0 || N % 16 != 0) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!aligned16(aq) || !aligned16(bq) || !aligned16(c)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_gemm_fp8(aq, bq, c, (int)M, (int)N, (int)K, scale_a * scale_b,
+                                        trans_b != 0, static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+// Shared device-side vocabulary for the gfx950 kernels: vector types, MFMA wrappers,
+// bf16 packing, cross-lane helpers.  Wave size is 64 everywhere.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tyr {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+constexpr int kWave = 64;
+
+// ---- MFMA (dense, f32 accumulate) -------------------------------------------------
+// Operand layout facts used throughout (lane = l, wave64):
+//   32x32x16 bf16 : A lane holds row  l%32, k = 8*(l/32)+[0,8) ; B lane holds col l%32, same k.
+//                   D reg r (0..15)  <-> row 8*(r/4) + 4*(l/32) + r%4, col l%32.
+//   16x16x32 bf16 : A lane holds row  l%16, k = 8*(l/16)+[0,8) ; B lane holds col l%16, same k.
+//                   D reg r (0..3)   <-> row 4*(l/16) + r, col l%16.
+//   32x32x64 fp8  : as 32x32x16 with 32 bytes of k per lane (k = 32*(l/32)+[0,32)).
+// Only "A and B use the same k <-> (lane group, slot) map" matters for correctness of a
+// product, so kernels are free to permute k as long as both operands agree.
+
+__device__ __forceinline__ f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma_16x16x32_bf16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+// FP8 E4M3 x E4M3 (format code 0 on both operands), scales fixed at 1 (unscaled encoding).
+__device__ __forceinline__ f32x16 mfma_32x32x64_e4m3(i32x8 a, i32x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// ---- bf16 packing -----------------------------------------------------------------
+// Round-to-nearest-even f32 -> bf16 pair (v_cvt_pk_bf16_f32); lo goes to bits [15:0].
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    bf16x2 r = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
+
+// ---- cross-lane -------------------------------------------------------------------
+// Value held by lane l^32.
+__device__ __forceinline__ float xor32(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    // s.x: lanes 0-31 keep their own value, lanes 32-63 receive lanes 0-31.
+    // s.y: lanes 0-31 receive lanes 32-63, lanes 32-63 keep their own value.
+    uint32_t other = (threadIdx.x & 32) ? s.x : s.y;
+    return __builtin_bit_cast(float, other);
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, s.x), __builtin_bit_cast(float, s.y));
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, s.x) + __builtin_bit_cast(float, s.y);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- 16-byte global / LDS moves ----------------------------------------------------
+__device__ __forceinline__ u32x4 ld_global_16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ u32x2 ld_global_8(const void* p) { return *reinterpret_cast<const u32x2*>(p); }
+__device__ __forceinline__ void st_global_16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+__device__ __forceinline__ void st_global_8(void* p, u32x2 v) { *reinterpret_cast<u32x2*>(p) = v; }
+
+// 8x8 transpose of 16-bit elements held as 8 rows of 4 dwords: out[c] holds column c
+// (8 elements = 4 dwords, element r in half (r&1) of dword r/2).
+__device__ __forceinline__ void transpose8x8_b16(const u32x4 (&in)[8], u32x4 (&out)[8]) {
+#pragma unroll
+    for (int c2 = 0; c2 < 4; ++c2) {      // column pair (2*c2, 2*c2+1) lives in dword c2 of every row
+        u32x4 lo, hi;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {     // output dword j packs rows 2j, 2j+1
+            uint32_t x0 = in[2 * j][c2], x1 = in[2 * j + 1][c2];
+            lo[j] = __builtin_amdgcn_perm(x1, x0, 0x05040100u);   // [x0.lo16, x1.lo16]
+            hi[j] = __builtin_amdgcn_perm(x1, x0, 0x07060302u);   // [x0.hi16, x1.hi16]
+        }
+        out[2 * c2] = lo;
+        out[2 * c2 + 1] = hi;
+    }
+}
+
+// Grid remap for the 8 XCDs of an MI355X: consecutive workgroup ids are dealt round-robin
+// to the XCDs, each with its own L2.  This returns a logical id such that the workgroups
+// that land on one XCD cover one contiguous range of logical ids (so neighbours in the
+// logical order share an L2).  Falls back to the identity when n is not a multiple of 8.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t n) {
+    if (n % 8u) return pid;
+    return (pid % 8u) * (n / 8u) + pid / 8u;
+}
+
+}  // namespace tyr

@@ -1,0 +1,325 @@
+// Flash-attention forward for gfx950 (bf16 in, f32 softmax, bf16 O + f32 LSE).
+//
+// Arithmetic contract of the reference (order of operations):
+//   Tyr/GPU/Kernels/MhaH100.lean:102-128   S = Q K^T ; S *= scale ; online softmax ; P -> bf16 ;
+//                                          O += P V ; O /= l ; LSE = ln l + m ; O -> bf16
+//   Tyr/GPU/Codegen/Macros.lean:121-163    m' = max(m,rowmax) ; alpha = exp(m-m') ; O,l *= alpha ;
+//                                          P = exp(S-m') ; l += rowsum P(f32)
+//   causal semantics: key j visible to query i iff j <= i (cc/src/tyr.cpp:2578-2585, is_causal).
+// exp is evaluated as exp2 with log2(e) folded into the scale; O is rescaled only on tiles where
+// some row maximum of the wave moved (alpha == 1 otherwise).
+//
+// Work decomposition.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave
+// owns 32 rows.  Keys/values stream through LDS in tiles of 64 rows, two stages deep, fetched
+// into registers one tile ahead.
+//
+// The products are computed transposed so the softmax never leaves the lane:
+//   S^T (64 kv x 32 q)  = K_tile (row operand, from LDS)  x  Q^T (column operand, registers)
+//   O^T (D x 32 q)     += V_tile^T (row operand, from LDS) x  P^T (column operand, registers)
+// With the 32x32 MFMA every lane then holds one query column (l%32) of S^T and O^T: the row
+// max/sum are register reductions plus one exchange with lane l^32, the rescale is a per-lane
+// scalar, and the exponentials of S^T are already in the register slots the second product
+// wants for P^T.  The k index of the second product is a permutation of the kv rows (fixed by
+// the accumulator layout of the first); V is written to LDS transposed with the same
+// permutation, 8x(D/32) blocks transposed in registers on the way in.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace tyr {
+
+namespace fa {
+constexpr int BM = 128, BN = 64, THREADS = 256;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+template <int D>
+struct Cfg {
+    static constexpr int K_ROW = D * 2 + 16;        // bytes per K row in LDS (padded)
+    static constexpr int K_TILE = BN * K_ROW;
+    static constexpr int V_ROW = BN * 2 + 16;       // bytes per V^T row (one d, 64 kv) in LDS
+    static constexpr int V_TILE = D * V_ROW;
+    static constexpr int STAGE = K_TILE + V_TILE;
+    static constexpr int LDS = 2 * STAGE;
+    static constexpr int KCH = D / 8;               // 16-byte chunks per K row
+    static constexpr int K_PER_THREAD = BN * KCH / THREADS;
+    static constexpr int DW = D / 32;               // d columns per V loader unit (8 kv x DW d)
+    static constexpr int KSTEPS = D / 16;           // MFMA k-steps of Q K^T
+    static constexpr int DT = D / 32;               // 32-row tiles of O^T
+};
+
+// kv row (within the 64-row tile) held in slot p of 16-byte chunk cu of a V^T row.
+// cu = 4*T + 2*s + g : S^T sub-tile T, k-step s of the second product, lane half g.
+__device__ __forceinline__ int v_chunk_row(int cu, int p) {
+    return (cu >> 2) * 32 + ((cu >> 1) & 1) * 16 + (cu & 1) * 4 + (p >> 2) * 8 + (p & 3);
+}
+}  // namespace fa
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
+    const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
+    uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2) {
+    using namespace fa;
+    using C = Cfg<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int r = lane & 31, g = lane >> 5;
+
+    // workgroup -> (head, query tile).  Heads are dealt to the 8 XCDs so that all query tiles of a
+    // head run on one XCD (shared K/V in its L2); within a head the longest (last) causal tiles
+    // are issued first.
+    int bh, qt;
+    {
+        const int id = blockIdx.x;
+        int tr;
+        if ((BH & 7) == 0) {
+            const int xcd = id & 7, slot = id >> 3;
+            bh = (slot / ntq) * 8 + xcd;
+            tr = slot % ntq;
+        } else {
+            bh = id / ntq;
+            tr = id % ntq;
+        }
+        qt = CAUSAL ? ntq - 1 - tr : tr;
+    }
+    const int q0 = qt * BM;
+    const int qw0 = q0 + w * 32;                 // first query row of this wave
+    const size_t head_off = (size_t)bh * N * D;
+    const uint16_t* Qh = Q + head_off;
+    const uint16_t* Kh = Kp + head_off;
+    const uint16_t* Vh = Vp + head_off;
+
+    const int kv_end = CAUSAL ? min(N, q0 + BM) : N;
+    const int nkv = (kv_end + BN - 1) / BN;
+
+    // ---- Q^T fragments: lane holds row qw0+r, columns 16i + 8g + [0,8)
+    bf16x8 qf[C::KSTEPS];
+    {
+        const int qrow = min(qw0 + r, N - 1);
+        const uint16_t* qp = Qh + (size_t)qrow * D + g * 8;
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i)
+            qf[i] = __builtin_bit_cast(bf16x8, ld_global_16(qp + i * 16));
+    }
+
+    // ---- K/V tile loaders
+    u32x4 rk[C::K_PER_THREAD];
+    uint32_t rv[8][C::DW / 2];                   // 8 kv rows x DW bf16
+    const int v_cu = t & 7, v_db = t >> 3;       // V unit: chunk cu, d columns v_db*DW + [0,DW)
+
+    auto load_tile = [&](int j0) {
+#pragma unroll
+        for (int i = 0; i < C::K_PER_THREAD; ++i) {
+            const int c = t + THREADS * i;
+            const int row = min(j0 + c / C::KCH, N - 1);
+            rk[i] = ld_global_16(Kh + (size_t)row * D + (c % C::KCH) * 8);
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int row = min(j0 + v_chunk_row(v_cu, p), N - 1);
+            const uint16_t* vp = Vh + (size_t)row * D + v_db * C::DW;
+            if (C::DW == 4) {
+                const u32x2 x = ld_global_8(vp);
+                rv[p][0] = x.x;
+                rv[p][C::DW / 2 - 1] = x.y;
+            } else {
+                rv[p][0] = *reinterpret_cast<const uint32_t*>(vp);
+            }
+        }
+    };
+
+    auto store_tile = [&](int stage) {
+        unsigned char* Ks = lds + stage * C::STAGE;
+        unsigned char* Vs = Ks + C::K_TILE;
+#pragma unroll
+        for (int i = 0; i < C::K_PER_THREAD; ++i) {
+            const int c = t + THREADS * i;
+            *reinterpret_cast<u32x4*>(Ks + (c / C::KCH) * C::K_ROW + (c % C::KCH) * 16) = rk[i];
+        }
+        // transpose 8 kv x DW d -> DW rows of 8 kv (16 bytes each)
+#pragma unroll
+        for (int h = 0; h < C::DW / 2; ++h) {
+            u32x4 lo, hi;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                lo[jj] = __builtin_amdgcn_perm(rv[2 * jj + 1][h], rv[2 * jj][h], 0x05040100u);
+                hi[jj] = __builtin_amdgcn_perm(rv[2 * jj + 1][h], rv[2 * jj][h], 0x07060302u);
+            }
+            const int d = v_db * C::DW + 2 * h;
+            *reinterpret_cast<u32x4*>(Vs + d * C::V_ROW + v_cu * 16) = lo;
+            *reinterpret_cast<u32x4*>(Vs + (d + 1) * C::V_ROW + v_cu * 16) = hi;
+        }
+    };
+
+    f32x16 oacc[C::DT];
+#pragma unroll
+    for (int i = 0; i < C::DT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[i][e] = 0.0f;
+    float m2 = -INFINITY;      // running row maximum, in log2 units (score * scale * log2 e)
+    float lsum = 0.0f;         // this lane's share of the running row sum
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    const int k_off = r * C::K_ROW + g * 16;
+    const int v_off = r * C::V_ROW + g * 16;
+    const int qpos = qw0 + r;
+
+    for (int j = 0; j < nkv; ++j) {
+        const int stage = j & 1;
+        const int j0 = j * BN;
+        if (j + 1 < nkv) load_tile(j0 + BN);
+
+        // tiles entirely above the diagonal of this wave's rows contribute nothing
+        const bool wave_active = !CAUSAL || (j0 <= qw0 + 31);
+        if (wave_active) {
+            const unsigned char* Ks = lds + stage * C::STAGE + k_off;
+            const unsigned char* Vs = lds + stage * C::STAGE + C::K_TILE + v_off;
+            const bool t1_active = !CAUSAL || (j0 + 32 <= qw0 + 31);
+
+            f32x16 sacc[2];
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) sacc[T][e] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < C::KSTEPS; ++i) {
+                const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(Ks + i * 32);
+                sacc[0] = mfma_32x32x16_bf16(k0, qf[i], sacc[0]);
+            }
+            if (t1_active) {
+#pragma unroll
+                for (int i = 0; i < C::KSTEPS; ++i) {
+                    const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(Ks + 32 * C::K_ROW + i * 32);
+                    sacc[1] = mfma_32x32x16_bf16(k1, qf[i], sacc[1]);
+                }
+            }
+
+            // ---- mask (diagonal tiles, ragged tail) -- register e of sub-tile T is kv row
+            //      j0 + 32T + 8(e/4) + 4g + e%4
+            const bool need_mask = (CAUSAL && (j0 + BN - 1 > qw0)) || (j0 + BN > N);
+            if (need_mask) {
+                const int lim = CAUSAL ? min(qpos, N - 1) : N - 1;   // largest visible kv row
+                const int base = j0 + 4 * g;
+#pragma unroll
+                for (int T = 0; T < 2; ++T)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
+                        if (kv > lim) sacc[T][e] = -INFINITY;
+                    }
+            }
+            if (!t1_active) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) sacc[1][e] = -INFINITY;
+            }
+
+            // ---- online softmax on this lane's query column
+            float mx = sacc[0][0];
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[T][e]);
+            mx = max_xor32(mx);
+            const float m2new = fmaxf(m2, mx * scale_log2);
+            const float alpha = fast_exp2(m2 - m2new);
+            if (__builtin_amdgcn_ballot_w64(m2new > m2) != 0) {
+#pragma unroll
+                for (int i = 0; i < C::DT; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+            }
+            m2 = m2new;
+            float psum = 0.0f;
+            bf16x8 pf[2][2];
+#pragma unroll
+            for (int T = 0; T < 2; ++T) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    u32x4 pk;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const float p0 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj], scale_log2, -m2new));
+                        const float p1 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj + 1], scale_log2, -m2new));
+                        psum += p0 + p1;
+                        pk[jj] = pack_bf16(p0, p1);
+                    }
+                    pf[T][s] = __builtin_bit_cast(bf16x8, pk);
+                }
+            }
+            lsum = lsum * alpha + psum;
+
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (2 * s) * 16);
+                    oacc[dt] = mfma_32x32x16_bf16(vf, pf[0][s], oacc[dt]);
+                }
+            }
+            if (t1_active) {
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (4 + 2 * s) * 16);
+                        oacc[dt] = mfma_32x32x16_bf16(vf, pf[1][s], oacc[dt]);
+                    }
+                }
+            }
+        }
+
+        if (j + 1 < nkv) store_tile(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- finalize: O /= l, LSE = ln l + m
+    const float ltot = sum_xor32(lsum);
+    const float inv = 1.0f / ltot;
+    if (qpos < N) {
+        uint16_t* orow = O + head_off + (size_t)qpos * D;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                u32x2 v;
+                v.x = pack_bf16(oacc[dt][4 * q4 + 0] * inv, oacc[dt][4 * q4 + 1] * inv);
+                v.y = pack_bf16(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv);
+                st_global_8(orow + dt * 32 + q4 * 8 + g * 4, v);
+            }
+        }
+        if (LSE != nullptr && g == 0) LSE[(size_t)bh * N + qpos] = logf(ltot) + m2 * LN2;
+    }
+}
+
+int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
+                          int H, int N, int D, int causal, float scale, hipStream_t stream) {
+    using namespace fa;
+    const int BH = B * H;
+    const int ntq = (N + BM - 1) / BM;
+    dim3 grid((unsigned)(BH * ntq)), block(THREADS);
+    const float scale_log2 = scale * LOG2E;
+    auto Qp = static_cast<const uint16_t*>(q);
+    auto Kp = static_cast<const uint16_t*>(k);
+    auto Vp = static_cast<const uint16_t*>(v);
+    auto Op = static_cast<uint16_t*>(o);
+#define TYR_FA_LAUNCH(DD, CC)                                                                    \
+    do {                                                                                         \
+        static const hipError_t attr = hipFuncSetAttribute(                                      \
+            reinterpret_cast<const void*>(&flash_attn_fwd_kernel<DD, CC>),                       \
+            hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DD>::LDS);                           \
+        if (attr != hipSuccess) return -1;                                                       \
+        hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC>), grid, block, Cfg<DD>::LDS, stream,   \
+                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2);                         \
+    } while (0)
+    if (D == 128) { if (causal) TYR_FA_LAUNCH(128, true); else TYR_FA_LAUNCH(128, false); }
+    else          { if (causal) TYR_FA_LAUNCH(64, true);  else TYR_FA_LAUNCH(64, false); }
+#undef TYR_FA_LAUNCH
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace tyr

@@ -1,0 +1,224 @@
+// FP8 (OCP E4M3) GEMM for gfx950 with per-tensor scales:
+//   C[M,N] = bf16( scale * sum_k e4m3(Aq[m,k]) * e4m3(Bq[k,n]) ),  scale = scale_a * scale_b,
+// f32 accumulation on the 32x32x64 F8F6F4 MFMA (both operands format E4M3, block scales off),
+// the scalar applied once in the epilogue.
+//
+// Arithmetic contract of the reference: Tyr/GPU/Kernels/PrecisionGemm.lean:97-115,178-189
+// (e4m3 x e4m3 -> f32 -> bf16) and Tyr/GPU/Kernels/GemmCommon.lean:135-144 (one scalar
+// multiplied into the f32 accumulator tile before the store).
+//
+// Same skeleton as the bf16 GEMM: 256x256 output tile per 4-wave workgroup, K in slices of
+// 128 bytes, k-contiguous padded LDS rows for both operands, two LDS stages with register
+// prefetch, one barrier per slice.  For B stored [K,N] the loader transposes 16(k) x 8(n) byte
+// blocks in registers (two levels of v_perm_b32) on the way to LDS.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace tyr {
+
+namespace gemm8 {
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int ROW_BYTES = BK + 16;               // 144
+constexpr int TILE_BYTES = BM * ROW_BYTES;
+constexpr int LDS_BYTES = 4 * TILE_BYTES;
+constexpr int THREADS = 256;
+constexpr int GROUP_M = 4;
+}  // namespace gemm8
+
+// 4x4 byte transpose: o[c] = {x0.byte c, x1.byte c, x2.byte c, x3.byte c}.
+__device__ __forceinline__ void transpose4x4_b8(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3,
+                                                uint32_t (&o)[4]) {
+    const uint32_t t0 = __builtin_amdgcn_perm(x1, x0, 0x05010400u);  // x0.b0 x1.b0 x0.b1 x1.b1
+    const uint32_t t1 = __builtin_amdgcn_perm(x1, x0, 0x07030602u);  // x0.b2 x1.b2 x0.b3 x1.b3
+    const uint32_t t2 = __builtin_amdgcn_perm(x3, x2, 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(x3, x2, 0x07030602u);
+    o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+template <bool TRANS_B, bool EDGE>
+__global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, int tiles_m, int tiles_n, float scale) {
+    using namespace gemm8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = w >> 1, wn = w & 1;
+
+    const uint32_t nblk = (uint32_t)tiles_m * (uint32_t)tiles_n;
+    const uint32_t pid = xcd_remap(blockIdx.x, nblk);
+    const uint32_t per_group = GROUP_M * (uint32_t)tiles_n;
+    const uint32_t grp = pid / per_group;
+    const uint32_t first_m = grp * GROUP_M;
+    const uint32_t gsz = min((uint32_t)tiles_m - first_m, (uint32_t)GROUP_M);
+    const int tm = (int)(first_m + (pid % per_group) % gsz);
+    const int tn = (int)((pid % per_group) / gsz);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    u32x4 ra[8];
+    u32x4 rb[8];   // TRANS_B: 8 chunks of 16 B.  Otherwise viewed as 16 rows x 8 B.
+
+    auto load_slice = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = t + THREADS * i;
+            const int row = c >> 3, kc = c & 7;
+            const int gm = m0 + row, gk = k0 + kc * 16;
+            if (!EDGE || (gm < M && gk < K))
+                ra[i] = ld_global_16(A + (size_t)gm * K + gk);
+            else
+                ra[i] = u32x4{0, 0, 0, 0};
+        }
+        if (TRANS_B) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = t + THREADS * i;
+                const int row = c >> 3, kc = c & 7;
+                const int gn = n0 + row, gk = k0 + kc * 16;
+                if (!EDGE || (gn < N && gk < K))
+                    rb[i] = ld_global_16(B + (size_t)gn * K + gk);
+                else
+                    rb[i] = u32x4{0, 0, 0, 0};
+            }
+        } else {
+            const int kb = t & 7, nb = t >> 3;
+            const int gn = n0 + nb * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {       // rows 2i and 2i+1 of the 16(k) x 8(n) block
+                u32x2 lo = {0, 0}, hi = {0, 0};
+                const int gk = k0 + kb * 16 + 2 * i;
+                if (!EDGE || (gk < K && gn < N)) lo = ld_global_8(B + (size_t)gk * N + gn);
+                if (!EDGE || (gk + 1 < K && gn < N)) hi = ld_global_8(B + (size_t)(gk + 1) * N + gn);
+                rb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+            }
+        }
+    };
+
+    auto store_slice = [&](int stage) {
+        unsigned char* As = lds + stage * 2 * TILE_BYTES;
+        unsigned char* Bs = As + TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = t + THREADS * i;
+            *reinterpret_cast<u32x4*>(As + (c >> 3) * ROW_BYTES + (c & 7) * 16) = ra[i];
+        }
+        if (TRANS_B) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = t + THREADS * i;
+                *reinterpret_cast<u32x4*>(Bs + (c >> 3) * ROW_BYTES + (c & 7) * 16) = rb[i];
+            }
+        } else {
+            const int kb = t & 7, nb = t >> 3;
+            // row k (0..15) of the block: dwords (n0..3, n4..7) = rb[k/2][2*(k&1) + {0,1}]
+            u32x4 out[8];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {          // n half: columns 4h..4h+3
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {      // k group: rows 4j..4j+3 -> output dword j
+                    uint32_t o[4];
+                    transpose4x4_b8(rb[2 * j][h], rb[2 * j][2 + h], rb[2 * j + 1][h], rb[2 * j + 1][2 + h], o);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) out[4 * h + c][j] = o[c];
+                }
+            }
+#pragma unroll
+            for (int nn = 0; nn < 8; ++nn)
+                *reinterpret_cast<u32x4*>(Bs + (nb * 8 + nn) * ROW_BYTES + kb * 16) = out[nn];
+        }
+    };
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int KT = (K + BK - 1) / BK;
+    load_slice(0);
+    store_slice(0);
+    __syncthreads();
+
+    const int a_off = (wm * 128 + r) * ROW_BYTES + g * 32;
+    const int b_off = (wn * 128 + r) * ROW_BYTES + g * 32;
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int stage = kt & 1;
+        if (kt + 1 < KT) load_slice((kt + 1) * BK);
+
+        const unsigned char* As = lds + stage * 2 * TILE_BYTES + a_off;
+        const unsigned char* Bs = lds + stage * 2 * TILE_BYTES + TILE_BYTES + b_off;
+#pragma unroll
+        for (int s = 0; s < BK / 64; ++s) {
+            i32x8 af[4], bf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x4 a0 = *reinterpret_cast<const u32x4*>(As + i * 32 * ROW_BYTES + s * 64);
+                const u32x4 a1 = *reinterpret_cast<const u32x4*>(As + i * 32 * ROW_BYTES + s * 64 + 16);
+                const u32x4 b0 = *reinterpret_cast<const u32x4*>(Bs + i * 32 * ROW_BYTES + s * 64);
+                const u32x4 b1 = *reinterpret_cast<const u32x4*>(Bs + i * 32 * ROW_BYTES + s * 64 + 16);
+                af[i] = i32x8{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                bf[i] = i32x8{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[j], af[i], acc[i][j]);
+        }
+
+        if (kt + 1 < KT) store_slice(stage ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int gm = m0 + wm * 128 + i * 32 + r;
+        if (EDGE && gm >= M) continue;
+        uint16_t* crow = C + (size_t)gm * N;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int gn = n0 + wn * 128 + j * 32 + q4 * 8 + g * 4;
+                if (EDGE && gn >= N) continue;
+                u32x2 v;
+                v.x = pack_bf16(acc[i][j][q4 * 4 + 0] * scale, acc[i][j][q4 * 4 + 1] * scale);
+                v.y = pack_bf16(acc[i][j][q4 * 4 + 2] * scale, acc[i][j][q4 * 4 + 3] * scale);
+                st_global_8(crow + gn, v);
+            }
+        }
+    }
+}
+
+int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
+                    int trans_b, hipStream_t stream) {
+    using namespace gemm8;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const bool edge = (M % BM) || (N % BN) || (K % BK);
+    dim3 grid((unsigned)(tiles_m * tiles_n)), block(THREADS);
+    auto A = static_cast<const uint8_t*>(aq);
+    auto Bp = static_cast<const uint8_t*>(bq);
+    auto Cp = static_cast<uint16_t*>(c);
+#define TYR_GEMM8_LAUNCH(TB, ED)                                                                  \
+    do {                                                                                          \
+        static const hipError_t attr = hipFuncSetAttribute(                                       \
+            reinterpret_cast<const void*>(&gemm_fp8_kernel<TB, ED>),                              \
+            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);                               \
+        if (attr != hipSuccess) return -1;                                                        \
+        hipLaunchKernelGGL((gemm_fp8_kernel<TB, ED>), grid, block, LDS_BYTES, stream, A, Bp, Cp,  \
+                           M, N, K, tiles_m, tiles_n, scale);                                     \
+    } while (0)
+    if (trans_b) { if (edge) TYR_GEMM8_LAUNCH(true, true); else TYR_GEMM8_LAUNCH(true, false); }
+    else         { if (edge) TYR_GEMM8_LAUNCH(false, true); else TYR_GEMM8_LAUNCH(false, false); }
+#undef TYR_GEMM8_LAUNCH
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace tyr

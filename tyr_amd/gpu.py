@@ -1,0 +1,154 @@
+"""Host-side mirror of the Lean entry points ``Tyr.GPU.GFX950.*`` for torch tensors.
+
+Same names, argument meaning and error behaviour as the Lean declarations in
+``tyr_amd/lean/Tyr/GPU/GFX950.lean`` (which bind ``lean_tyr_gpu_*`` in
+``csrc/lean_shim.cpp``): outputs are freshly allocated and returned, every tensor argument
+is checked the way the reference's generated launcher checks it
+(Tyr/GPU/Codegen/Attribute.lean:334-336: device, contiguity, rank <= 4) and a failed
+check or a negative status from the C ABI raises ``TyrGpuError`` -- the analogue of the
+``IO.userError`` the Lean wrappers return.  torch is used for device memory and the
+current stream only; all arithmetic happens in ``libtyr_hip.so``.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+
+
+class TyrGpuError(RuntimeError):
+    """Raised where the Lean wrapper would return ``IO.userError msg``."""
+
+
+def library_path() -> str:
+    return _lib.LIB_PATH
+
+
+def _check(t: torch.Tensor, name: str, dtype, ndim: int | None = None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TyrGpuError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise TyrGpuError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise TyrGpuError(f"{name} must be contiguous")
+    if t.dim() > 4:
+        raise TyrGpuError(f"{name} must have dim <= 4")
+    if ndim is not None and t.dim() != ndim:
+        raise TyrGpuError(f"{name} must have dim == {ndim}")
+    if t.dtype != dtype:
+        raise TyrGpuError(f"{name} must have dtype {dtype}")
+
+
+def _raise(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = _lib.load().tyr_hip_strerror(rc).decode()
+        raise TyrGpuError(f"{what}: {msg} (status {rc})")
+
+
+def _stream(stream) -> int:
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, torch.cuda.Stream):
+        return stream.cuda_stream
+    return int(stream)
+
+
+def device_info(device: int = 0) -> dict:
+    L = _lib.load()
+    name = ctypes.create_string_buffer(64)
+    cu, lds, clk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    hbm = ctypes.c_size_t()
+    _raise(L.tyr_hip_device_info(device, name, 64, ctypes.byref(cu), ctypes.byref(lds), ctypes.byref(clk),
+                                 ctypes.byref(hbm)), "device_info")
+    return {"arch": name.value.decode(), "compute_units": cu.value, "lds_bytes_per_cu": lds.value,
+            "clock_mhz": clk.value, "hbm_bytes": hbm.value}
+
+
+def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, stream=None):
+    """O, LSE = flashAttnFwd q k v causal scale.  q,k,v bf16 [B,H,N,D] -> (bf16 [B,H,N,D], f32 [B,H,N])."""
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _check(t, n, torch.bfloat16, 4)
+    if k.shape != q.shape or v.shape != q.shape:
+        raise TyrGpuError("q, k, v must have the same shape [B, H, N, D]")
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    o = torch.empty_like(q)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    rc = _lib.load().tyr_hip_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                            lse.data_ptr(), B, H, N, D, int(bool(causal)), float(scale),
+                                            _stream(stream))
+    _raise(rc, "flashAttnFwd")
+    return o, lse
+
+
+def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len: int | None = None,
+               stream=None):
+    """O, LSE = gqaDecode q k v scale numSplits.
+
+    q bf16 [B,Hq,1,D]; k, v bf16 [B,Hkv,Lmax,D] (the preallocated cache); the first ``kv_len``
+    rows (default all) of every (batch, kv head) are attended to.  -> (bf16 [B,Hq,1,D], f32 [B,Hq]).
+    """
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _check(t, n, torch.bfloat16, 4)
+    B, Hq, one, D = q.shape
+    if one != 1:
+        raise TyrGpuError("q must have shape [B, Hq, 1, D]")
+    if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D:
+        raise TyrGpuError("k, v must have shape [B, Hkv, L, D]")
+    Hkv, Lmax = k.shape[1], k.shape[2]
+    L = Lmax if kv_len is None else int(kv_len)
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    o = torch.empty_like(q)
+    lse = torch.empty((B, Hq), dtype=torch.float32, device=q.device)
+    nbytes = lib.tyr_hip_gqa_decode_workspace_bytes(B, Hq, max(Hkv, 1), max(L, 1), D, int(num_splits))
+    ws = torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=q.device)
+    rc = lib.tyr_hip_gqa_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                B, Hq, Hkv, L, D, Lmax, float(scale), int(num_splits), ws.data_ptr(),
+                                ws.numel(), _stream(stream))
+    _raise(rc, "gqaDecode")
+    return o, lse
+
+
+def gemm_bf16(a, b, trans_b: bool = False, stream=None):
+    """C = gemmBf16 a b.  a bf16 [M,K]; b bf16 [K,N] (or [N,K] with trans_b) -> bf16 [M,N]."""
+    _check(a, "a", torch.bfloat16, 2)
+    _check(b, "b", torch.bfloat16, 2)
+    M, K = a.shape
+    N, Kb = (b.shape[0], b.shape[1]) if trans_b else (b.shape[1], b.shape[0])
+    if Kb != K:
+        raise TyrGpuError("a and b have mismatched inner dimensions")
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    rc = _lib.load().tyr_hip_gemm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, int(bool(trans_b)),
+                                       _stream(stream))
+    _raise(rc, "gemmBf16")
+    return c
+
+
+def gemm_fp8(aq, bq, scale_a: float, scale_b: float, trans_b: bool = False, stream=None):
+    """C = gemmFp8 aq bq scaleA scaleB.  aq e4m3 [M,K]; bq e4m3 [K,N] (or [N,K]) -> bf16 [M,N]."""
+    _check(aq, "a", torch.float8_e4m3fn, 2)
+    _check(bq, "b", torch.float8_e4m3fn, 2)
+    M, K = aq.shape
+    N, Kb = (bq.shape[0], bq.shape[1]) if trans_b else (bq.shape[1], bq.shape[0])
+    if Kb != K:
+        raise TyrGpuError("a and b have mismatched inner dimensions")
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=aq.device)
+    rc = _lib.load().tyr_hip_gemm_fp8(aq.data_ptr(), bq.data_ptr(), c.data_ptr(), M, N, K, float(scale_a),
+                                      float(scale_b), int(bool(trans_b)), _stream(stream))
+    _raise(rc, "gemmFp8")
+    return c
+
+
+def quantize_e4m3(x: torch.Tensor):
+    """Per-tensor absmax quantisation used by the harness: s = absmax/448, xq = e4m3fn(x / s)."""
+    s = float(x.abs().max()) / 448.0
+    if s == 0.0:
+        s = 1.0
+    xq = (x.float() / s).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return xq, s
