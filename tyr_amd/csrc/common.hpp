@@ -49,25 +49,28 @@ __device__ __forceinline__ float bf16_lo(uint32_t u) { return __builtin_bit_cast
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
 
 // ---- cross-lane -------------------------------------------------------------------
-// Value held by lane l^32.
+// Value held by lane l^32.  v_permlane32_swap exchanges lanes 32-63 of its first register with
+// lanes 0-31 of its second; fed the same value twice, the partner's value is in the first
+// result for the upper half-wave and in the second for the lower half-wave.  (Selecting per
+// half also stays right if the compiler assigns both operands to one register, in which case
+// either result holds the partner's value.)
 __device__ __forceinline__ float xor32(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    // s.x: lanes 0-31 keep their own value, lanes 32-63 receive lanes 0-31.
-    // s.y: lanes 0-31 receive lanes 32-63, lanes 32-63 keep their own value.
     uint32_t other = (threadIdx.x & 32) ? s.x : s.y;
     return __builtin_bit_cast(float, other);
 }
-__device__ __forceinline__ float max_xor32(float x) {
+// Value held by lane l^16 (same construction with v_permlane16_swap on 16-lane rows).
+__device__ __forceinline__ float xor16(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
-    u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, s.x), __builtin_bit_cast(float, s.y));
+    u32x2 s = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    uint32_t other = (threadIdx.x & 16) ? s.x : s.y;
+    return __builtin_bit_cast(float, other);
 }
-__device__ __forceinline__ float sum_xor32(float x) {
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    u32x2 s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return __builtin_bit_cast(float, s.x) + __builtin_bit_cast(float, s.y);
-}
+__device__ __forceinline__ float max_xor32(float x) { return fmaxf(x, xor32(x)); }
+__device__ __forceinline__ float sum_xor32(float x) { return x + xor32(x); }
+__device__ __forceinline__ float max_xor16(float x) { return fmaxf(x, xor16(x)); }
+__device__ __forceinline__ float sum_xor16(float x) { return x + xor16(x); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -35,17 +35,6 @@ struct Buf {
 };
 }  // namespace dec
 
-__device__ __forceinline__ float max_xor16(float x) {
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    u32x2 s = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, s.x), __builtin_bit_cast(float, s.y));
-}
-__device__ __forceinline__ float sum_xor16(float x) {
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    u32x2 s = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    return __builtin_bit_cast(float, s.x) + __builtin_bit_cast(float, s.y);
-}
-
 __global__ __launch_bounds__(dec::THREADS) void gqa_decode_split_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     float* __restrict__ part_o, float* __restrict__ part_m, float* __restrict__ part_l,
