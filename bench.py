@@ -198,7 +198,21 @@ def wl_gemm_fp8(torch, tyr, steps, warmup, cpu):
     return res
 
 
+def wl_copy(torch, tyr, steps, warmup, cpu):
+    """Counter calibration only: a plain device copy of exactly 1 GiB (reads 2^30 B, writes 2^30 B)."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    wall, ms = time_steps(torch, lambda: dst.copy_(src), steps, warmup)
+    gbs = 2.0 * n / (ms * 1e-3) / 1e9
+    return {"metric": "copy GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+            "dtype": "u8", "config": {"workload": "device-to-device copy of 1 GiB (counter calibration)"},
+            "roofline": {"bound": "hbm", "kernel": "torch elementwise copy", "achieved": gbs, "peak": PEAK["hbm"],
+                         "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": 2.0 * n}}
+
+
 WORKLOADS = {"attn_fwd_causal": wl_attn, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16, "gemm_fp8": wl_gemm_fp8}
+CALIBRATION = {"copy_1gib": wl_copy}
 
 
 def main() -> int:
@@ -206,7 +220,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="attn_fwd_causal", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="attn_fwd_causal", choices=sorted(WORKLOADS) + sorted(CALIBRATION))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
     args = ap.parse_args()
@@ -222,7 +236,9 @@ def main() -> int:
     torch.cuda.set_device(0)
     info = tyr_amd.device_info(0)
 
-    head = WORKLOADS[args.workload](torch, tyr_amd, args.steps, args.warmup, not args.no_cpu)
+    if args.workload in CALIBRATION:
+        args.no_extra = True
+    head = {**WORKLOADS, **CALIBRATION}[args.workload](torch, tyr_amd, args.steps, args.warmup, not args.no_cpu)
     line = {
         "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms_per_step"], 5),

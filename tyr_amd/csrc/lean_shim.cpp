@@ -1,0 +1,173 @@
+// Lean-facing wrappers over the C ABI in include/tyr_hip.h.
+//
+// These are the symbols the `@[extern]` declarations in lean/Tyr/GPU/GFX950.lean bind.  They
+// follow the conventions of the reference's FFI:
+//   * tensor arguments are *borrowed* Lean external objects wrapping a c10::TensorImpl
+//     (`borrowTensor`, cc/src/tyr.cpp:127-148); results are handed to Lean with `giveTensor`
+//     (cc/src/tyr.cpp:152-160);
+//   * implicit `{B H N D : UInt64}` binders arrive first as unboxed uint64_t
+//     (cc/src/tyr.cpp:3913-3918), Lean `Float` is C double, `Bool` is uint8_t
+//     (cc/src/tyr.cpp:2571-2572);
+//   * errors never cross the boundary as C++ exceptions: they become
+//     `IO.userError msg` (Tyr/GPU/Codegen/Attribute.lean:373-386), with the launcher's own
+//     messages "<p> must be a CUDA tensor" / "<p> must be contiguous" / "<p> must have dim <= 4"
+//     (Tyr/GPU/Codegen/Attribute.lean:334-336);
+//   * a pair is returned as `lean_alloc_ctor(0, 2, 0)` (cc/src/tyr.cpp:4275-4283) inside
+//     `lean_io_result_mk_ok`; the trailing IO world token is declared explicitly.
+//
+// The file is compiled into libTyrC only where <lean/lean.h> and LibTorch headers exist (the
+// reference's `make -C cc`); nothing else in this library depends on Lean or torch.
+#if defined(__has_include)
+#if __has_include(<lean/lean.h>) && __has_include(<torch/torch.h>)
+#define TYR_HAVE_LEAN 1
+#endif
+#endif
+
+#ifdef TYR_HAVE_LEAN
+#include <lean/lean.h>
+#include <torch/torch.h>
+
+#include <cmath>
+#include <string>
+
+#include "../../include/tyr_hip.h"
+
+// Provided by the reference's cc/src/tyr.cpp (same library).
+torch::Tensor borrowTensor(b_lean_obj_arg o);
+lean_object* giveTensor(torch::Tensor t);
+
+namespace {
+
+lean_object* io_error(const std::string& msg) {
+    return lean_io_result_mk_error(lean_mk_io_user_error(lean_mk_string(msg.c_str())));
+}
+
+// The reference launcher's three checks, plus the dtype the kernel expects.
+bool check(const torch::Tensor& t, const char* name, c10::ScalarType dt, std::string& err) {
+    if (!t.is_cuda()) { err = std::string(name) + " must be a CUDA tensor"; return false; }
+    if (!t.is_contiguous()) { err = std::string(name) + " must be contiguous"; return false; }
+    if (t.dim() > 4) { err = std::string(name) + " must have dim <= 4"; return false; }
+    if (t.scalar_type() != dt) { err = std::string(name) + " has the wrong dtype"; return false; }
+    return true;
+}
+
+lean_object* pair_result(torch::Tensor a, torch::Tensor b) {
+    lean_object* p = lean_alloc_ctor(0, 2, 0);
+    lean_ctor_set(p, 0, giveTensor(std::move(a)));
+    lean_ctor_set(p, 1, giveTensor(std::move(b)));
+    return lean_io_result_mk_ok(p);
+}
+
+lean_object* status_error(const char* what, int rc) {
+    return io_error(std::string(what) + ": " + tyr_hip_strerror(rc));
+}
+
+}  // namespace
+
+extern "C" {
+
+// flashAttnFwd {B H N D} q k v causal scale stream : IO (T #[B,H,N,D] x T #[B,H,N])
+lean_object* lean_tyr_gpu_flash_attn_fwd(uint64_t B, uint64_t H, uint64_t N, uint64_t D,
+                                         b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                         uint8_t causal, double scale, uint64_t stream,
+                                         lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err))
+            return io_error(err);
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)H, (int64_t)N}, q_.options().dtype(torch::kFloat32));
+        const int rc = tyr_hip_flash_attn_fwd(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                              lse.data_ptr<float>(), B, H, N, D, causal, (float)scale,
+                                              reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnFwd", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gqaDecode {B Hq Hkv L D} q k v scale numSplits stream : IO (T #[B,Hq,1,D] x T #[B,Hq])
+lean_object* lean_tyr_gpu_gqa_decode(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                                     b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v, double scale,
+                                     uint64_t num_splits, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err))
+            return io_error(err);
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)Hq}, q_.options().dtype(torch::kFloat32));
+        const size_t ws_bytes = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
+        auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
+        const int rc = tyr_hip_gqa_decode(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                          lse.data_ptr<float>(), B, Hq, Hkv, L, D, /*kv_stride=*/L,
+                                          (float)scale, num_splits, ws.data_ptr(), ws_bytes,
+                                          reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gqaDecode", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gemmBf16 {M N K} a b stream : IO (T #[M,N])
+lean_object* lean_tyr_gpu_gemm_bf16(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a,
+                                    b_lean_obj_arg b, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b);
+        std::string err;
+        if (!check(a_, "a", torch::kBFloat16, err) || !check(b_, "b", torch::kBFloat16, err))
+            return io_error(err);
+        auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options());
+        const int rc = tyr_hip_gemm_bf16(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, 0,
+                                         reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gemmBf16", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gemmBf16NT {M N K} a (b : T #[N,K]) stream : IO (T #[M,N])   -- the N x K form of tiledAccumulator
+lean_object* lean_tyr_gpu_gemm_bf16_nt(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a,
+                                       b_lean_obj_arg b, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b);
+        std::string err;
+        if (!check(a_, "a", torch::kBFloat16, err) || !check(b_, "b", torch::kBFloat16, err))
+            return io_error(err);
+        auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options());
+        const int rc = tyr_hip_gemm_bf16(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, 1,
+                                         reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gemmBf16NT", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gemmFp8 {M N K} a b scaleA scaleB stream : IO (T #[M,N])
+lean_object* lean_tyr_gpu_gemm_fp8(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a,
+                                   b_lean_obj_arg b, double scale_a, double scale_b, uint64_t stream,
+                                   lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b);
+        std::string err;
+        if (!check(a_, "a", torch::kFloat8_e4m3fn, err) || !check(b_, "b", torch::kFloat8_e4m3fn, err))
+            return io_error(err);
+        auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options().dtype(torch::kBFloat16));
+        const int rc = tyr_hip_gemm_fp8(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, (float)scale_a,
+                                        (float)scale_b, 0, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gemmFp8", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+}  // extern "C"
+#endif  // TYR_HAVE_LEAN

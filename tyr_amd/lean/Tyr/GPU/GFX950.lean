@@ -1,0 +1,74 @@
+/-
+  Tyr.GPU.GFX950 — entry points of the MI355X (gfx950 / CDNA4) kernel library.
+
+  These are plain `@[extern]` opaques in the style of `Tyr/Torch.lean:1058-1082`
+  (`scaledDotProductAttentionGQA`), not `@[gpu_kernel]` DSL kernels: the kernels behind
+  them are hand-written HIP, so no `GpuArch` constructor is involved and none of the
+  exhaustive matches on `GpuArch` change.  Shapes are carried in the types; the implicit
+  `UInt64` binders reach the C side first, unboxed, in binder order.
+
+  Unlike the generated `X.launch … : IO Unit` launchers (`Tyr/GPU/Codegen/Attribute.lean:390-437`),
+  which mutate caller-allocated outputs behind Lean's back, these return freshly allocated
+  tensors in `IO`.
+
+  C side: `tyr_amd/csrc/lean_shim.cpp` (wrappers) over `include/tyr_hip.h` (C ABI).
+-/
+import Tyr.Basic
+import Tyr.GPU.Codegen.TileTypes
+
+namespace Tyr.GPU.GFX950
+
+open torch
+open Tyr.GPU.Codegen (CudaStream)
+
+/-- Capabilities of the one target this library is built for. Nothing matches on it. -/
+structure Capabilities where
+  arch : String := "gfx950"
+  waveSize : Nat := 64
+  computeUnits : Nat := 256
+  ldsBytesPerCU : Nat := 163840
+  /-- dense bf16 MFMA tile shapes used by the kernels (M, N, K) -/
+  mfmaBf16 : List (Nat × Nat × Nat) := [(32, 32, 16), (16, 16, 32)]
+  /-- dense FP8 (OCP E4M3) MFMA tile shape -/
+  mfmaFp8 : List (Nat × Nat × Nat) := [(32, 32, 64)]
+  fp8Format : String := "OCP e4m3fn (bias 7, max 448, no inf)"
+  deriving Repr
+
+def capabilities : Capabilities := {}
+
+/-- Flash-attention forward. `q k v : bf16 [B,H,N,D]`, `D ∈ {64,128}`.
+    Returns `(O : bf16 [B,H,N,D], LSE : f32 [B,H,N])` with `LSE = ln Σ_j exp(scale · qᵢ·kⱼ)`.
+    GPU twin of `nn.scaled_dot_product_attention` (`Tyr/Torch.lean:665-671`). -/
+@[extern "lean_tyr_gpu_flash_attn_fwd"]
+opaque flashAttnFwd {B H N D : UInt64} (q k v : @& T #[B, H, N, D]) (causal : Bool) (scale : Float)
+    (stream : CudaStream) : IO (T #[B, H, N, D] × T #[B, H, N])
+
+/-- GQA decode attention, one query token per sequence, split-KV with an LSE combine pass.
+    `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D = 128`,
+    query head `h` reads kv head `h / (Hq/Hkv)`; `numSplits = 0` lets the library choose.
+    GPU twin of `nn.scaledDotProductAttentionGQAQKV` with `is_causal = false`
+    (`Tyr/Torch.lean:1070-1082`, caller `Tyr/Model/Qwen/Attention.lean:199-200`). -/
+@[extern "lean_tyr_gpu_gqa_decode"]
+opaque gqaDecode {B Hq Hkv L D : UInt64} (q : @& T #[B, Hq, 1, D]) (k v : @& T #[B, Hkv, L, D])
+    (scale : Float) (numSplits : UInt64) (stream : CudaStream) : IO (T #[B, Hq, 1, D] × T #[B, Hq])
+
+/-- `C = A · B`, bf16 operands, f32 accumulation, bf16 result; `b` is `K × N` row-major.
+    GPU twin of `nn.mm` (`Tyr/Torch.lean:546`). -/
+@[extern "lean_tyr_gpu_gemm_bf16"]
+opaque gemmBf16 {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (stream : CudaStream)
+    : IO (T #[M, N])
+
+/-- `C = A · Bᵀ` with `b` stored `N × K` (the operand layout of `tiledAccumulator`,
+    `Tyr/GPU/Kernels/GemmCommon.lean:22-56`). -/
+@[extern "lean_tyr_gpu_gemm_bf16_nt"]
+opaque gemmBf16NT {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[N, K]) (stream : CudaStream)
+    : IO (T #[M, N])
+
+/-- FP8 (e4m3fn) GEMM with per-tensor scales: `C = bf16 (scaleA · scaleB · (Aq · Bq))`.
+    Counterpart of `gemmFp8E4M3Fwd` / `tkH100Fp8ScaledGemmFwd`
+    (`Tyr/GPU/Kernels/PrecisionGemm.lean:97-115,178-189`). -/
+@[extern "lean_tyr_gpu_gemm_fp8"]
+opaque gemmFp8 {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (scaleA scaleB : Float)
+    (stream : CudaStream) : IO (T #[M, N])
+
+end Tyr.GPU.GFX950
