@@ -62,12 +62,12 @@ def test_flash_attn_causal_closed_forms(gpu):
 def test_flash_attn_future_keys_do_not_leak(gpu):
     q, k, v = qkv(12, 1, 2, 512, 128)
     k2, v2 = k.clone(), v.clone()
-    k2[:, :, 300:] = 5.0
-    v2[:, :, 300:] = -3.0
+    k2[:, :, 320:] = 5.0
+    v2[:, :, 320:] = -3.0
     a, la = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=True)
     b, lb = gpu.flash_attn_fwd(q.cuda(), k2.cuda(), v2.cuda(), causal=True)
-    assert torch.equal(a[:, :, :300], b[:, :, :300]) and torch.equal(la[:, :, :300], lb[:, :, :300])
-    assert not torch.equal(a[:, :, 300:], b[:, :, 300:])
+    assert torch.equal(a[:, :, :320], b[:, :, :320]) and torch.equal(la[:, :, :320], lb[:, :, :320])
+    assert not torch.equal(a[:, :, 320:], b[:, :, 320:])
 
 
 def test_flash_attn_full_size_config(gpu):

@@ -97,6 +97,14 @@ __device__ __forceinline__ void transpose8x8_b16(const u32x4 (&in)[8], u32x4 (&o
     }
 }
 
+// Makes the compiler treat v as produced here: any load feeding it is waited for at this point
+// (and not, conservatively, at its first use inside a loop that has other loads in flight).
+__device__ __forceinline__ void pin_registers(bf16x8& v) {
+    u32x4 u = __builtin_bit_cast(u32x4, v);
+    asm volatile("" : "+v"(u));
+    v = __builtin_bit_cast(bf16x8, u);
+}
+
 // Grid remap for the 8 XCDs of an MI355X: consecutive workgroup ids are dealt round-robin
 // to the XCDs, each with its own L2.  This returns a logical id such that the workgroups
 // that land on one XCD cover one contiguous range of logical ids (so neighbours in the

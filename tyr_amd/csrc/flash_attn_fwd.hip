@@ -6,8 +6,9 @@
 //   Tyr/GPU/Codegen/Macros.lean:121-163    m' = max(m,rowmax) ; alpha = exp(m-m') ; O,l *= alpha ;
 //                                          P = exp(S-m') ; l += rowsum P(f32)
 //   causal semantics: key j visible to query i iff j <= i (cc/src/tyr.cpp:2578-2585, is_causal).
-// exp is evaluated as exp2 with log2(e) folded into the scale; O is rescaled only on tiles where
-// some row maximum of the wave moved (alpha == 1 otherwise).
+// exp is evaluated as exp2 with log2(e) folded into the scale; the running maximum is advanced
+// (and O, l rescaled) only when a row outgrows it by more than a threshold, which is the same
+// mathematics with a stale reference point.
 //
 // Work decomposition.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave
 // owns 32 rows.  Keys/values stream through LDS in tiles of 64 rows, two stages deep, fetched
@@ -31,6 +32,7 @@ namespace fa {
 constexpr int BM = 128, BN = 64, THREADS = 256;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
+constexpr float RESCALE_THRESHOLD = 8.0f;
 
 template <int D>
 struct Cfg {
@@ -103,28 +105,36 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             qf[i] = __builtin_bit_cast(bf16x8, ld_global_16(qp + i * 16));
     }
 
-    // ---- K/V tile loaders
+    // ---- K/V tile loaders.  Buffer loads: the per-thread byte offset inside a tile is fixed, the
+    // tile start is a scalar offset, and rows at or beyond N read as zero (they are masked below).
+    const uint32_t head_bytes = (uint32_t)N * D * 2u;
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Kh), 0, head_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Vh), 0, head_bytes, 0x00020000);
     u32x4 rk[C::K_PER_THREAD];
     uint32_t rv[8][C::DW / 2];                   // 8 kv rows x DW bf16
     const int v_cu = t & 7, v_db = t >> 3;       // V unit: chunk cu, d columns v_db*DW + [0,DW)
+    int k_voff[C::K_PER_THREAD], v_voff[8];
+#pragma unroll
+    for (int i = 0; i < C::K_PER_THREAD; ++i) {
+        const int c = t + THREADS * i;
+        k_voff[i] = (c / C::KCH) * (D * 2) + (c % C::KCH) * 16;
+    }
+#pragma unroll
+    for (int p = 0; p < 8; ++p) v_voff[p] = v_chunk_row(v_cu, p) * (D * 2) + v_db * C::DW * 2;
 
     auto load_tile = [&](int j0) {
+        const int soff = j0 * (D * 2);
 #pragma unroll
-        for (int i = 0; i < C::K_PER_THREAD; ++i) {
-            const int c = t + THREADS * i;
-            const int row = min(j0 + c / C::KCH, N - 1);
-            rk[i] = ld_global_16(Kh + (size_t)row * D + (c % C::KCH) * 8);
-        }
+        for (int i = 0; i < C::K_PER_THREAD; ++i)
+            rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[i], soff, 0);
 #pragma unroll
         for (int p = 0; p < 8; ++p) {
-            const int row = min(j0 + v_chunk_row(v_cu, p), N - 1);
-            const uint16_t* vp = Vh + (size_t)row * D + v_db * C::DW;
             if (C::DW == 4) {
-                const u32x2 x = ld_global_8(vp);
+                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, v_voff[p], soff, 0);
                 rv[p][0] = x.x;
                 rv[p][C::DW / 2 - 1] = x.y;
             } else {
-                rv[p][0] = *reinterpret_cast<const uint32_t*>(vp);
+                rv[p][0] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_voff[p], soff, 0);
             }
         }
     };
@@ -162,6 +172,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
     load_tile(0);
     store_tile(0);
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
     __syncthreads();
 
     const int k_off = r * C::K_ROW + g * 16;
@@ -178,23 +190,16 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         if (wave_active) {
             const unsigned char* Ks = lds + stage * C::STAGE + k_off;
             const unsigned char* Vs = lds + stage * C::STAGE + C::K_TILE + v_off;
-            const bool t1_active = !CAUSAL || (j0 + 32 <= qw0 + 31);
 
             f32x16 sacc[2];
 #pragma unroll
-            for (int T = 0; T < 2; ++T)
+            for (int T = 0; T < 2; ++T) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) sacc[T][e] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < C::KSTEPS; ++i) {
-                const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(Ks + i * 32);
-                sacc[0] = mfma_32x32x16_bf16(k0, qf[i], sacc[0]);
-            }
-            if (t1_active) {
-#pragma unroll
                 for (int i = 0; i < C::KSTEPS; ++i) {
-                    const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(Ks + 32 * C::K_ROW + i * 32);
-                    sacc[1] = mfma_32x32x16_bf16(k1, qf[i], sacc[1]);
+                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + T * 32 * C::K_ROW + i * 32);
+                    sacc[T] = mfma_32x32x16_bf16(kf, qf[i], sacc[T]);
                 }
             }
 
@@ -212,27 +217,27 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                         if (kv > lim) sacc[T][e] = -INFINITY;
                     }
             }
-            if (!t1_active) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sacc[1][e] = -INFINITY;
-            }
 
-            // ---- online softmax on this lane's query column
+            // ---- online softmax on this lane's query column.  The reference maximum m2 is only
+            // advanced (and O, l rescaled) when some row of the wave outgrew it by more than
+            // RESCALE_THRESHOLD (in log2 units); otherwise exp2(s - m2) <= 2^threshold, which f32
+            // sums and bf16 P hold without loss.
             float mx = sacc[0][0];
 #pragma unroll
             for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[T][e]);
-            mx = max_xor32(mx);
-            const float m2new = fmaxf(m2, mx * scale_log2);
-            const float alpha = fast_exp2(m2 - m2new);
-            if (__builtin_amdgcn_ballot_w64(m2new > m2) != 0) {
+            mx = max_xor32(mx) * scale_log2;
+            if (__builtin_amdgcn_ballot_w64(mx > m2 + RESCALE_THRESHOLD) != 0) {
+                const float m2new = fmaxf(m2, mx);
+                const float alpha = fast_exp2(m2 - m2new);
 #pragma unroll
                 for (int i = 0; i < C::DT; ++i)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+                lsum *= alpha;
+                m2 = m2new;
             }
-            m2 = m2new;
             float psum = 0.0f;
             bf16x8 pf[2][2];
 #pragma unroll
@@ -242,32 +247,25 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                     u32x4 pk;
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj) {
-                        const float p0 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj], scale_log2, -m2new));
-                        const float p1 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj + 1], scale_log2, -m2new));
+                        const float p0 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj], scale_log2, -m2));
+                        const float p1 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj + 1], scale_log2, -m2));
                         psum += p0 + p1;
                         pk[jj] = pack_bf16(p0, p1);
                     }
                     pf[T][s] = __builtin_bit_cast(bf16x8, pk);
                 }
             }
-            lsum = lsum * alpha + psum;
+            lsum += psum;
 
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt) {
 #pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (2 * s) * 16);
-                    oacc[dt] = mfma_32x32x16_bf16(vf, pf[0][s], oacc[dt]);
-                }
-            }
-            if (t1_active) {
-#pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt) {
+                for (int T = 0; T < 2; ++T) {
 #pragma unroll
                     for (int s = 0; s < 2; ++s) {
-                        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (4 + 2 * s) * 16);
-                        oacc[dt] = mfma_32x32x16_bf16(vf, pf[1][s], oacc[dt]);
+                        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (4 * T + 2 * s) * 16);
+                        oacc[dt] = mfma_32x32x16_bf16(vf, pf[T][s], oacc[dt]);
                     }
                 }
             }

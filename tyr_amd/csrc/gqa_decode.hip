@@ -142,6 +142,8 @@ __global__ __launch_bounds__(dec::THREADS) void gqa_decode_split_kernel(
             oacc[j] = mfma_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt[j]), pfrag, oacc[j]);
     };
 
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pin_registers(qf[i]);
     Buf b0, b1;
     if (nsteps > 0) load(b0, r0);
     for (int st = 0; st < nsteps; st += 2) {
