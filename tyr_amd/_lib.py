@@ -5,7 +5,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtyr_hip.so")
+# TYR_HIP_LIBRARY overrides the location (e.g. to try an experimental build); there is still no fallback.
+LIB_PATH = os.environ.get("TYR_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libtyr_hip.so")
 
 # every symbol include/tyr_hip.h declares
 SYMBOLS = (

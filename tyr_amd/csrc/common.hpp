@@ -105,6 +105,15 @@ __device__ __forceinline__ void pin_registers(bf16x8& v) {
     v = __builtin_bit_cast(bf16x8, u);
 }
 
+// ds_read_b64_tr_b16: transposing LDS read.  Within each block of 16 lanes, lane 4q+p receives
+// element p (16 bits) of the 8-byte pieces addressed by lanes q, q+4, q+8, q+12 of the block.
+__device__ __forceinline__ bf16x4 ds_read_tr16(const void* lds_ptr) {
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(lds_ptr));
+    return __builtin_bit_cast(bf16x4, v);
+}
+
 // Grid remap for the 8 XCDs of an MI355X: consecutive workgroup ids are dealt round-robin
 // to the XCDs, each with its own L2.  This returns a logical id such that the workgroups
 // that land on one XCD cover one contiguous range of logical ids (so neighbours in the

@@ -21,8 +21,13 @@
 // max/sum are register reductions plus one exchange with lane l^32, the rescale is a per-lane
 // scalar, and the exponentials of S^T are already in the register slots the second product
 // wants for P^T.  The k index of the second product is a permutation of the kv rows (fixed by
-// the accumulator layout of the first); V is written to LDS transposed with the same
-// permutation, 8x(D/32) blocks transposed in registers on the way in.
+// the accumulator layout of the first).
+//
+// K and V tiles sit in LDS row-major (one 2D-byte row per kv position, 16-byte chunks XOR-swizzled
+// so that neither access pattern has bank conflicts).  K fragments are plain 16-byte reads (lane =
+// kv row).  V^T fragments come from ds_read_b64_tr_b16: within each 16-lane block, lane 4q+p
+// receives element p of the 8-byte pieces addressed by lanes q, q+4, q+8, q+12 -- so four lanes
+// pointing at 4 consecutive d of 4 kv rows hand every lane "its" d for those 4 rows.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -36,24 +41,24 @@ constexpr float RESCALE_THRESHOLD = 8.0f;
 
 template <int D>
 struct Cfg {
-    static constexpr int K_ROW = D * 2 + 16;        // bytes per K row in LDS (padded)
-    static constexpr int K_TILE = BN * K_ROW;
-    static constexpr int V_ROW = BN * 2 + 16;       // bytes per V^T row (one d, 64 kv) in LDS
-    static constexpr int V_TILE = D * V_ROW;
+    static constexpr int ROW = D * 2;               // bytes per K or V row in LDS
+    static constexpr int KCH = D / 8;               // 16-byte chunks per row
+    static constexpr int K_TILE = BN * ROW;
+    static constexpr int V_TILE = BN * ROW;
     static constexpr int STAGE = K_TILE + V_TILE;
     static constexpr int LDS = 2 * STAGE;
-    static constexpr int KCH = D / 8;               // 16-byte chunks per K row
-    static constexpr int K_PER_THREAD = BN * KCH / THREADS;
-    static constexpr int DW = D / 32;               // d columns per V loader unit (8 kv x DW d)
+    static constexpr int PER_THREAD = BN * KCH / THREADS;   // 16-byte chunks per thread per tile
     static constexpr int KSTEPS = D / 16;           // MFMA k-steps of Q K^T
     static constexpr int DT = D / 32;               // 32-row tiles of O^T
 };
 
-// kv row (within the 64-row tile) held in slot p of 16-byte chunk cu of a V^T row.
-// cu = 4*T + 2*s + g : S^T sub-tile T, k-step s of the second product, lane half g.
-__device__ __forceinline__ int v_chunk_row(int cu, int p) {
-    return (cu >> 2) * 32 + ((cu >> 1) & 1) * 16 + (cu & 1) * 4 + (p >> 2) * 8 + (p & 3);
-}
+// Swizzles (chunk index within a row -> stored chunk index).
+//   K: lanes of one read hold 16 consecutive rows and the same chunk -> spread over all chunks.
+//   V: one transposing read touches 4 consecutive rows x 64 bytes per lane-group pair -> move each
+//      row of a group of 4 to a different 64-byte quarter... (for D = 64 rows are 128 bytes and the
+//      quarter index has one bit less).
+template <int D> __device__ __forceinline__ int k_swz(int row, int c) { return c ^ (row & (Cfg<D>::KCH - 1)); }
+template <int D> __device__ __forceinline__ int v_swz(int row, int c) { return c ^ (((row & 3) << 2) & (Cfg<D>::KCH - 1)); }
 }  // namespace fa
 
 template <int D, bool CAUSAL>
@@ -110,56 +115,31 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint32_t head_bytes = (uint32_t)N * D * 2u;
     const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Kh), 0, head_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Vh), 0, head_bytes, 0x00020000);
-    u32x4 rk[C::K_PER_THREAD];
-    uint32_t rv[8][C::DW / 2];                   // 8 kv rows x DW bf16
-    const int v_cu = t & 7, v_db = t >> 3;       // V unit: chunk cu, d columns v_db*DW + [0,DW)
-    int k_voff[C::K_PER_THREAD], v_voff[8];
+    u32x4 rk[C::PER_THREAD], rv[C::PER_THREAD];
+    int g_voff[C::PER_THREAD], k_soff[C::PER_THREAD], v_soff[C::PER_THREAD];
 #pragma unroll
-    for (int i = 0; i < C::K_PER_THREAD; ++i) {
-        const int c = t + THREADS * i;
-        k_voff[i] = (c / C::KCH) * (D * 2) + (c % C::KCH) * 16;
+    for (int i = 0; i < C::PER_THREAD; ++i) {
+        const int n = t + THREADS * i;
+        const int row = n / C::KCH, c = n % C::KCH;
+        g_voff[i] = row * C::ROW + c * 16;                              // coalesced: 16 B per lane along a row
+        k_soff[i] = row * C::ROW + k_swz<D>(row, c) * 16;
+        v_soff[i] = C::K_TILE + row * C::ROW + v_swz<D>(row, c) * 16;
     }
-#pragma unroll
-    for (int p = 0; p < 8; ++p) v_voff[p] = v_chunk_row(v_cu, p) * (D * 2) + v_db * C::DW * 2;
 
     auto load_tile = [&](int j0) {
-        const int soff = j0 * (D * 2);
+        const int soff = j0 * C::ROW;
 #pragma unroll
-        for (int i = 0; i < C::K_PER_THREAD; ++i)
-            rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[i], soff, 0);
+        for (int i = 0; i < C::PER_THREAD; ++i) rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, g_voff[i], soff, 0);
 #pragma unroll
-        for (int p = 0; p < 8; ++p) {
-            if (C::DW == 4) {
-                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, v_voff[p], soff, 0);
-                rv[p][0] = x.x;
-                rv[p][C::DW / 2 - 1] = x.y;
-            } else {
-                rv[p][0] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_voff[p], soff, 0);
-            }
-        }
+        for (int i = 0; i < C::PER_THREAD; ++i) rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, g_voff[i], soff, 0);
     };
 
     auto store_tile = [&](int stage) {
-        unsigned char* Ks = lds + stage * C::STAGE;
-        unsigned char* Vs = Ks + C::K_TILE;
+        unsigned char* base = lds + stage * C::STAGE;
 #pragma unroll
-        for (int i = 0; i < C::K_PER_THREAD; ++i) {
-            const int c = t + THREADS * i;
-            *reinterpret_cast<u32x4*>(Ks + (c / C::KCH) * C::K_ROW + (c % C::KCH) * 16) = rk[i];
-        }
-        // transpose 8 kv x DW d -> DW rows of 8 kv (16 bytes each)
+        for (int i = 0; i < C::PER_THREAD; ++i) *reinterpret_cast<u32x4*>(base + k_soff[i]) = rk[i];
 #pragma unroll
-        for (int h = 0; h < C::DW / 2; ++h) {
-            u32x4 lo, hi;
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                lo[jj] = __builtin_amdgcn_perm(rv[2 * jj + 1][h], rv[2 * jj][h], 0x05040100u);
-                hi[jj] = __builtin_amdgcn_perm(rv[2 * jj + 1][h], rv[2 * jj][h], 0x07060302u);
-            }
-            const int d = v_db * C::DW + 2 * h;
-            *reinterpret_cast<u32x4*>(Vs + d * C::V_ROW + v_cu * 16) = lo;
-            *reinterpret_cast<u32x4*>(Vs + (d + 1) * C::V_ROW + v_cu * 16) = hi;
-        }
+        for (int i = 0; i < C::PER_THREAD; ++i) *reinterpret_cast<u32x4*>(base + v_soff[i]) = rv[i];
     };
 
     f32x16 oacc[C::DT];
@@ -176,8 +156,22 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
     __syncthreads();
 
-    const int k_off = r * C::K_ROW + g * 16;
-    const int v_off = r * C::V_ROW + g * 16;
+    // K fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g.
+    int k_roff[C::KSTEPS];
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) k_roff[i] = r * C::ROW + k_swz<D>(r, 2 * i + g) * 16;
+    // V^T fragment (d tile dt; rows 32T + 16s + 8h + 4g + [0,4)): as a source lane of the transposing
+    // read this lane points at row 4g + (lane%16)/4 of that group, 8 bytes at d = 32dt + 16(b&1) + 4(lane%4).
+    int v_roff[C::DT];
+    {
+        const int i16 = lane & 15, b16 = lane >> 4;
+        const int row = 4 * (b16 >> 1) + (i16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+            const int dcol = 32 * dt + 16 * (b16 & 1) + 4 * (i16 & 3);
+            v_roff[dt] = C::K_TILE + row * C::ROW + v_swz<D>(row, dcol >> 3) * 16 + (dcol & 7) * 2;
+        }
+    }
     const int qpos = qw0 + r;
 
     for (int j = 0; j < nkv; ++j) {
@@ -188,18 +182,33 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         // tiles entirely above the diagonal of this wave's rows contribute nothing
         const bool wave_active = !CAUSAL || (j0 <= qw0 + 31);
         if (wave_active) {
-            const unsigned char* Ks = lds + stage * C::STAGE + k_off;
-            const unsigned char* Vs = lds + stage * C::STAGE + C::K_TILE + v_off;
+            const unsigned char* St = lds + stage * C::STAGE;
 
+            // S^T = K Q^T.  LDS operand reads run one group of 4 fragments ahead of the MFMAs that
+            // consume them (two register groups, fenced so the order survives scheduling); the two
+            // 32-row sub-tiles alternate so consecutive MFMAs never chain on one accumulator.
             f32x16 sacc[2];
 #pragma unroll
-            for (int T = 0; T < 2; ++T) {
+            for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) sacc[T][e] = 0.0f;
+            {
+                constexpr int NG = C::KSTEPS / 2;        // groups of (2 k-steps x 2 sub-tiles)
+                bf16x8 kf[2][4];
+                auto read_group = [&](int grp, bf16x8 (&dst)[4]) {
 #pragma unroll
-                for (int i = 0; i < C::KSTEPS; ++i) {
-                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + T * 32 * C::K_ROW + i * 32);
-                    sacc[T] = mfma_32x32x16_bf16(kf, qf[i], sacc[T]);
+                    for (int u = 0; u < 4; ++u)
+                        dst[u] = *reinterpret_cast<const bf16x8*>(St + k_roff[2 * grp + (u >> 1)] + (u & 1) * 32 * C::ROW);
+                };
+                read_group(0, kf[0]);
+#pragma unroll
+                for (int grp = 0; grp < NG; ++grp) {
+                    if (grp + 1 < NG) read_group(grp + 1, kf[(grp + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        sacc[u & 1] = mfma_32x32x16_bf16(kf[grp & 1][u], qf[2 * grp + (u >> 1)], sacc[u & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
 
@@ -257,16 +266,28 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             }
             lsum += psum;
 
-            // ---- O^T += V^T P^T
+            // ---- O^T += V^T P^T, same read-ahead scheme: group c = (T, s) holds the DT row tiles
+            {
+                bf16x8 vf[2][C::DT];
+                auto read_group = [&](int c, bf16x8 (&dst)[C::DT]) {
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt) {
-#pragma unroll
-                for (int T = 0; T < 2; ++T) {
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + dt * 32 * C::V_ROW + (4 * T + 2 * s) * 16);
-                        oacc[dt] = mfma_32x32x16_bf16(vf, pf[T][s], oacc[dt]);
+                    for (int dt = 0; dt < C::DT; ++dt)
+                    {
+                        const unsigned char* p = St + v_roff[dt] + c * 16 * C::ROW;   // c = 2T + s: rows 16c + ...
+                        const bf16x4 lo = ds_read_tr16(p);
+                        const bf16x4 hi = ds_read_tr16(p + 8 * C::ROW);
+                        dst[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                     }
+                };
+                read_group(0, vf[0]);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (c + 1 < 4) read_group(c + 1, vf[(c + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+                        oacc[dt] = mfma_32x32x16_bf16(vf[c & 1][dt], pf[c >> 1][c & 1], oacc[dt]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
