@@ -105,6 +105,30 @@ __device__ __forceinline__ void pin_registers(bf16x8& v) {
     v = __builtin_bit_cast(bf16x8, u);
 }
 
+// Buffer resource (V#) for raw byte-addressed access to [base, base + bytes): loads beyond the
+// range return zero.
+__device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    return u32x4{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane i of the wave writes
+// lds_base + 16 i (lds_base wave-uniform); the source is rsrc.base + voffset + soffset.
+// Issued as opaque asm so that the compiler does not order later LDS reads behind it; the
+// caller waits with wait_vmcnt0() (and a barrier) before anyone reads the destination.  M0 is
+// written here; the compiler keeps nothing live in M0 on this target (it sets M0 itself right
+// before each of its own uses).
+__device__ __forceinline__ void load_global_to_lds_16(u32x4 rsrc, uint32_t lds_base, int voffset, int soffset) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen lds"
+        :
+        : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+        : "memory");
+}
+__device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // ds_read_b64_tr_b16: transposing LDS read.  Within each block of 16 lanes, lane 4q+p receives
 // element p (16 bits) of the 8-byte pieces addressed by lanes q, q+4, q+8, q+12 of the block.
 __device__ __forceinline__ bf16x4 ds_read_tr16(const void* lds_ptr) {

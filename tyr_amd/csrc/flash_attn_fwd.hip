@@ -11,8 +11,8 @@
 // mathematics with a stale reference point.
 //
 // Work decomposition.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave
-// owns 32 rows.  Keys/values stream through LDS in tiles of 64 rows, two stages deep, fetched
-// into registers one tile ahead.
+// owns 32 rows.  Keys/values stream through LDS in tiles of 64 rows, two stages deep, loaded
+// one tile ahead directly from global memory into LDS.
 //
 // The products are computed transposed so the softmax never leaves the lane:
 //   S^T (64 kv x 32 q)  = K_tile (row operand, from LDS)  x  Q^T (column operand, registers)
@@ -113,34 +113,33 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // ---- K/V tile loaders.  Buffer loads: the per-thread byte offset inside a tile is fixed, the
     // tile start is a scalar offset, and rows at or beyond N read as zero (they are masked below).
     const uint32_t head_bytes = (uint32_t)N * D * 2u;
-    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Kh), 0, head_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(Vh), 0, head_bytes, 0x00020000);
-    u32x4 rk[C::PER_THREAD], rv[C::PER_THREAD];
-    int g_voff[C::PER_THREAD], k_soff[C::PER_THREAD], v_soff[C::PER_THREAD];
+    const u32x4 k_rsrc = make_raw_rsrc(Kh, head_bytes);
+    const u32x4 v_rsrc = make_raw_rsrc(Vh, head_bytes);
+    // Tiles go from global memory straight into LDS (no register staging).  One load instruction
+    // of a wave fills 1 KiB of LDS linearly (lane i -> 16 bytes at base + 16 i); the swizzle is
+    // applied on the global side: the lane fetches the chunk that belongs at its LDS position.
+    constexpr int ROWS_PER_INST = 1024 / C::ROW;
+    int gk_voff[C::PER_THREAD], gv_voff[C::PER_THREAD];
 #pragma unroll
-    for (int i = 0; i < C::PER_THREAD; ++i) {
-        const int n = t + THREADS * i;
-        const int row = n / C::KCH, c = n % C::KCH;
-        g_voff[i] = row * C::ROW + c * 16;                              // coalesced: 16 B per lane along a row
-        k_soff[i] = row * C::ROW + k_swz<D>(row, c) * 16;
-        v_soff[i] = C::K_TILE + row * C::ROW + v_swz<D>(row, c) * 16;
+    for (int m = 0; m < C::PER_THREAD; ++m) {
+        const int row = (w * C::PER_THREAD + m) * ROWS_PER_INST + lane / C::KCH;
+        const int cpos = lane % C::KCH;                                 // chunk position in LDS
+        gk_voff[m] = row * C::ROW + k_swz<D>(row, cpos) * 16;          // swizzles are involutions
+        gv_voff[m] = row * C::ROW + v_swz<D>(row, cpos) * 16;
     }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PER_THREAD * 1024u);
 
-    auto load_tile = [&](int j0) {
+    auto issue_tile = [&](int stage, int j0) {
         const int soff = j0 * C::ROW;
+        const uint32_t kb = wave_dst + (uint32_t)stage * C::STAGE;
 #pragma unroll
-        for (int i = 0; i < C::PER_THREAD; ++i) rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, g_voff[i], soff, 0);
+        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(k_rsrc, kb + m * 1024, gk_voff[m], soff);
 #pragma unroll
-        for (int i = 0; i < C::PER_THREAD; ++i) rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, g_voff[i], soff, 0);
+        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(v_rsrc, kb + C::K_TILE + m * 1024, gv_voff[m], soff);
     };
-
-    auto store_tile = [&](int stage) {
-        unsigned char* base = lds + stage * C::STAGE;
-#pragma unroll
-        for (int i = 0; i < C::PER_THREAD; ++i) *reinterpret_cast<u32x4*>(base + k_soff[i]) = rk[i];
-#pragma unroll
-        for (int i = 0; i < C::PER_THREAD; ++i) *reinterpret_cast<u32x4*>(base + v_soff[i]) = rv[i];
-    };
+    // all of this wave's tile loads have landed in LDS
+    auto wait_tile = [&]() { wait_vmcnt0(); };
 
     f32x16 oacc[C::DT];
 #pragma unroll
@@ -150,10 +149,10 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     float m2 = -INFINITY;      // running row maximum, in log2 units (score * scale * log2 e)
     float lsum = 0.0f;         // this lane's share of the running row sum
 
-    load_tile(0);
-    store_tile(0);
+    issue_tile(0, 0);
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
+    wait_tile();
     __syncthreads();
 
     // K fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g.
@@ -177,7 +176,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     for (int j = 0; j < nkv; ++j) {
         const int stage = j & 1;
         const int j0 = j * BN;
-        if (j + 1 < nkv) load_tile(j0 + BN);
+        if (j + 1 < nkv) issue_tile(stage ^ 1, j0 + BN);
 
         // tiles entirely above the diagonal of this wave's rows contribute nothing
         const bool wave_active = !CAUSAL || (j0 <= qw0 + 31);
@@ -292,7 +291,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             }
         }
 
-        if (j + 1 < nkv) store_tile(stage ^ 1);
+        wait_tile();
         __syncthreads();
     }
 
