@@ -12,7 +12,9 @@
 //
 // Work decomposition.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave
 // owns 32 rows.  Keys/values stream through LDS in tiles of 64 rows, two stages deep, loaded
-// one tile ahead directly from global memory into LDS.
+// directly from global memory into LDS.  The loop is software-pipelined inside each wave: the
+// score MFMAs of tile j+1 are issued among the softmax instructions of tile j (so K runs one tile
+// ahead of V), which keeps the matrix pipe fed while the vector ALU does the exponentials.
 //
 // The products are computed transposed so the softmax never leaves the lane:
 //   S^T (64 kv x 32 q)  = K_tile (row operand, from LDS)  x  Q^T (column operand, registers)
@@ -45,8 +47,8 @@ struct Cfg {
     static constexpr int KCH = D / 8;               // 16-byte chunks per row
     static constexpr int K_TILE = BN * ROW;
     static constexpr int V_TILE = BN * ROW;
-    static constexpr int STAGE = K_TILE + V_TILE;
-    static constexpr int LDS = 2 * STAGE;
+    static constexpr int V_BASE = 2 * K_TILE;       // LDS: K stage 0, K stage 1, V stage 0, V stage 1
+    static constexpr int LDS = 2 * K_TILE + 2 * V_TILE;
     static constexpr int PER_THREAD = BN * KCH / THREADS;   // 16-byte chunks per thread per tile
     static constexpr int KSTEPS = D / 16;           // MFMA k-steps of Q K^T
     static constexpr int DT = D / 32;               // 32-row tiles of O^T
@@ -130,16 +132,16 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PER_THREAD * 1024u);
 
-    auto issue_tile = [&](int stage, int j0) {
-        const int soff = j0 * C::ROW;
-        const uint32_t kb = wave_dst + (uint32_t)stage * C::STAGE;
+    auto issue_k = [&](int stage, int j0) {
+        const uint32_t dst = wave_dst + (uint32_t)stage * C::K_TILE;
 #pragma unroll
-        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(k_rsrc, kb + m * 1024, gk_voff[m], soff);
-#pragma unroll
-        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(v_rsrc, kb + C::K_TILE + m * 1024, gv_voff[m], soff);
+        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(k_rsrc, dst + m * 1024, gk_voff[m], j0 * C::ROW);
     };
-    // all of this wave's tile loads have landed in LDS
-    auto wait_tile = [&]() { wait_vmcnt0(); };
+    auto issue_v = [&](int stage, int j0) {
+        const uint32_t dst = wave_dst + C::V_BASE + (uint32_t)stage * C::V_TILE;
+#pragma unroll
+        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(v_rsrc, dst + m * 1024, gv_voff[m], j0 * C::ROW);
+    };
 
     f32x16 oacc[C::DT];
 #pragma unroll
@@ -148,12 +150,6 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         for (int e = 0; e < 16; ++e) oacc[i][e] = 0.0f;
     float m2 = -INFINITY;      // running row maximum, in log2 units (score * scale * log2 e)
     float lsum = 0.0f;         // this lane's share of the running row sum
-
-    issue_tile(0, 0);
-#pragma unroll
-    for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
-    wait_tile();
-    __syncthreads();
 
     // K fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g.
     int k_roff[C::KSTEPS];
@@ -168,48 +164,62 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
             const int dcol = 32 * dt + 16 * (b16 & 1) + 4 * (i16 & 3);
-            v_roff[dt] = C::K_TILE + row * C::ROW + v_swz<D>(row, dcol >> 3) * 16 + (dcol & 7) * 2;
+            v_roff[dt] = C::V_BASE + row * C::ROW + v_swz<D>(row, dcol >> 3) * 16 + (dcol & 7) * 2;
         }
     }
     const int qpos = qw0 + r;
+    // number of kv tiles that intersect this wave's visible region
+    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / BN + 1) : nkv;
 
-    for (int j = 0; j < nkv; ++j) {
-        const int stage = j & 1;
+    constexpr int NG = C::KSTEPS / 2;            // S^T is built in NG groups of (2 k-steps x 2 sub-tiles)
+    auto read_k_group = [&](const unsigned char* Kt, int grp, bf16x8 (&dst)[4]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            dst[u] = *reinterpret_cast<const bf16x8*>(Kt + k_roff[2 * grp + (u >> 1)] + (u & 1) * 32 * C::ROW);
+    };
+    auto mfma_k_group = [&](f32x16 (&sacc)[2], int grp, const bf16x8 (&kf)[4]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sacc[u & 1] = mfma_32x32x16_bf16(kf[u], qf[2 * grp + (u >> 1)], sacc[u & 1]);
+    };
+    auto zero_s = [&](f32x16 (&sacc)[2]) {
+#pragma unroll
+        for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[T][e] = 0.0f;
+    };
+
+    // ---- prologue: K(0), V(0), K(1) in flight; S(0) computed on its own
+    issue_k(0, 0);
+    issue_v(0, 0);
+    if (nkv > 1) issue_k(1, BN);
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
+    wait_vmcnt0();
+    __syncthreads();
+
+    f32x16 sA[2], sB[2];
+    zero_s(sA);
+    {
+        bf16x8 kf[2][4];
+        read_k_group(lds, 0, kf[0]);
+#pragma unroll
+        for (int grp = 0; grp < NG; ++grp) {
+            if (grp + 1 < NG) read_k_group(lds, grp + 1, kf[(grp + 1) & 1]);
+            mfma_k_group(sA, grp, kf[grp & 1]);
+        }
+    }
+
+    // One kv tile: softmax and P V of tile j (scores in `cur`), overlapped with the score MFMAs of
+    // tile j+1 (into `nxt`).  K runs one tile ahead of V in LDS: at entry K(j+1) and V(j) are
+    // resident; K(j+2) and V(j+1) are requested here and awaited at the end.
+    auto tile_step = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2], int j) {
         const int j0 = j * BN;
-        if (j + 1 < nkv) issue_tile(stage ^ 1, j0 + BN);
+        if (j + 2 < nkv) issue_k(j & 1, j0 + 2 * BN);
+        if (j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
 
-        // tiles entirely above the diagonal of this wave's rows contribute nothing
-        const bool wave_active = !CAUSAL || (j0 <= qw0 + 31);
-        if (wave_active) {
-            const unsigned char* St = lds + stage * C::STAGE;
-
-            // S^T = K Q^T.  LDS operand reads run one group of 4 fragments ahead of the MFMAs that
-            // consume them (two register groups, fenced so the order survives scheduling); the two
-            // 32-row sub-tiles alternate so consecutive MFMAs never chain on one accumulator.
-            f32x16 sacc[2];
-#pragma unroll
-            for (int T = 0; T < 2; ++T)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sacc[T][e] = 0.0f;
-            {
-                constexpr int NG = C::KSTEPS / 2;        // groups of (2 k-steps x 2 sub-tiles)
-                bf16x8 kf[2][4];
-                auto read_group = [&](int grp, bf16x8 (&dst)[4]) {
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        dst[u] = *reinterpret_cast<const bf16x8*>(St + k_roff[2 * grp + (u >> 1)] + (u & 1) * 32 * C::ROW);
-                };
-                read_group(0, kf[0]);
-#pragma unroll
-                for (int grp = 0; grp < NG; ++grp) {
-                    if (grp + 1 < NG) read_group(grp + 1, kf[(grp + 1) & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        sacc[u & 1] = mfma_32x32x16_bf16(kf[grp & 1][u], qf[2 * grp + (u >> 1)], sacc[u & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
+        if (j < nkv_w) {
+            const unsigned char* Kt = lds + ((j + 1) & 1) * C::K_TILE;     // K(j+1) (stale on the last tile: unused)
+            const unsigned char* Vt = lds + (j & 1) * C::V_TILE;           // V(j), v_roff carries V_BASE
 
             // ---- mask (diagonal tiles, ragged tail) -- register e of sub-tile T is kv row
             //      j0 + 32T + 8(e/4) + 4g + e%4
@@ -222,19 +232,26 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        if (kv > lim) sacc[T][e] = -INFINITY;
+                        if (kv > lim) cur[T][e] = -INFINITY;
                     }
             }
 
-            // ---- online softmax on this lane's query column.  The reference maximum m2 is only
+            // ---- next tile's scores, first group, under the row-max reduction of this tile
+            bf16x8 kf[2][4];
+            zero_s(nxt);
+            read_k_group(Kt, 0, kf[0]);
+            read_k_group(Kt, 1, kf[1]);
+
+            // online softmax on this lane's query column.  The reference maximum m2 is only
             // advanced (and O, l rescaled) when some row of the wave outgrew it by more than
             // RESCALE_THRESHOLD (in log2 units); otherwise exp2(s - m2) <= 2^threshold, which f32
             // sums and bf16 P hold without loss.
-            float mx = sacc[0][0];
+            float mx = cur[0][0];
 #pragma unroll
             for (int T = 0; T < 2; ++T)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[T][e]);
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, cur[T][e]);
+            mfma_k_group(nxt, 0, kf[0]);
             mx = max_xor32(mx) * scale_log2;
             if (__builtin_amdgcn_ballot_w64(mx > m2 + RESCALE_THRESHOLD) != 0) {
                 const float m2new = fmaxf(m2, mx);
@@ -246,53 +263,59 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                 lsum *= alpha;
                 m2 = m2new;
             }
+
+            // ---- exponentials of this tile under the remaining score MFMAs of the next
             float psum = 0.0f;
             bf16x8 pf[2][2];
 #pragma unroll
-            for (int T = 0; T < 2; ++T) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    u32x4 pk;
-#pragma unroll
-                    for (int jj = 0; jj < 4; ++jj) {
-                        const float p0 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj], scale_log2, -m2));
-                        const float p1 = fast_exp2(fmaf(sacc[T][8 * s + 2 * jj + 1], scale_log2, -m2));
-                        psum += p0 + p1;
-                        pk[jj] = pack_bf16(p0, p1);
-                    }
-                    pf[T][s] = __builtin_bit_cast(bf16x8, pk);
+            for (int c = 0; c < 4; ++c) {                 // c = 2T + s : 8 scores each
+                const int T = c >> 1, sh = c & 1;
+                if (c + 1 < NG) {
+                    if (c + 2 < NG) read_k_group(Kt, c + 2, kf[c & 1]);
+                    mfma_k_group(nxt, c + 1, kf[(c + 1) & 1]);
                 }
+                u32x4 pk;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const float p0 = fast_exp2(fmaf(cur[T][8 * sh + 2 * jj], scale_log2, -m2));
+                    const float p1 = fast_exp2(fmaf(cur[T][8 * sh + 2 * jj + 1], scale_log2, -m2));
+                    psum += p0 + p1;
+                    pk[jj] = pack_bf16(p0, p1);
+                }
+                pf[T][sh] = __builtin_bit_cast(bf16x8, pk);
             }
             lsum += psum;
 
-            // ---- O^T += V^T P^T, same read-ahead scheme: group c = (T, s) holds the DT row tiles
+            // ---- O^T += V^T P^T; fragment reads run one group ahead.  Group c = (T, s).
             {
                 bf16x8 vf[2][C::DT];
-                auto read_group = [&](int c, bf16x8 (&dst)[C::DT]) {
+                auto read_v_group = [&](int c, bf16x8 (&dst)[C::DT]) {
 #pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-                    {
-                        const unsigned char* p = St + v_roff[dt] + c * 16 * C::ROW;   // c = 2T + s: rows 16c + ...
+                    for (int dt = 0; dt < C::DT; ++dt) {
+                        const unsigned char* p = Vt + v_roff[dt] + c * 16 * C::ROW;   // rows 16c + ...
                         const bf16x4 lo = ds_read_tr16(p);
                         const bf16x4 hi = ds_read_tr16(p + 8 * C::ROW);
                         dst[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                     }
                 };
-                read_group(0, vf[0]);
+                read_v_group(0, vf[0]);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    if (c + 1 < 4) read_group(c + 1, vf[(c + 1) & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
+                    if (c + 1 < 4) read_v_group(c + 1, vf[(c + 1) & 1]);
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
                         oacc[dt] = mfma_32x32x16_bf16(vf[c & 1][dt], pf[c >> 1][c & 1], oacc[dt]);
-                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
 
-        wait_tile();
+        wait_vmcnt0();
         __syncthreads();
+    };
+
+    for (int j = 0; j < nkv; j += 2) {
+        tile_step(sA, sB, j);
+        if (j + 1 < nkv) tile_step(sB, sA, j + 1);
     }
 
     // ---- finalize: O /= l, LSE = ln l + m
