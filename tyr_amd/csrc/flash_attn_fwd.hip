@@ -214,8 +214,10 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // resident; K(j+2) and V(j+1) are requested here and awaited at the end.
     auto tile_step = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2], int j) {
         const int j0 = j * BN;
+        // The two requests are issued apart (K here, V after the row-max reduction) so the waves of
+        // a CU do not all queue on the texture path at once.
         if (j + 2 < nkv) issue_k(j & 1, j0 + 2 * BN);
-        if (j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
+        if (j >= nkv_w && j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
 
         if (j < nkv_w) {
             const unsigned char* Kt = lds + ((j + 1) & 1) * C::K_TILE;     // K(j+1) (stale on the last tile: unused)
@@ -263,6 +265,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                 lsum *= alpha;
                 m2 = m2new;
             }
+
+            if (j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
 
             // ---- exponentials of this tile under the remaining score MFMAs of the next
             float psum = 0.0f;
