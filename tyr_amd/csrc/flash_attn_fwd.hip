@@ -271,6 +271,16 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             // ---- exponentials of this tile under the remaining score MFMAs of the next
             float psum = 0.0f;
             bf16x8 pf[2][2];
+            bf16x8 vf[2][C::DT];
+            auto read_v_group = [&](int c, bf16x8 (&dst)[C::DT]) {
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt) {
+                    const unsigned char* p = Vt + v_roff[dt] + c * 16 * C::ROW;   // rows 16c + ...
+                    const bf16x4 lo = ds_read_tr16(p);
+                    const bf16x4 hi = ds_read_tr16(p + 8 * C::ROW);
+                    dst[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+            };
 #pragma unroll
             for (int c = 0; c < 4; ++c) {                 // c = 2T + s : 8 scores each
                 const int T = c >> 1, sh = c & 1;
@@ -278,6 +288,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                     if (c + 2 < NG) read_k_group(Kt, c + 2, kf[c & 1]);
                     mfma_k_group(nxt, c + 1, kf[(c + 1) & 1]);
                 }
+                if (c == 3) read_v_group(0, vf[0]);       // first V^T fragments arrive under the last exponentials
                 u32x4 pk;
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) {
@@ -292,17 +303,6 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
             // ---- O^T += V^T P^T; fragment reads run one group ahead.  Group c = (T, s).
             {
-                bf16x8 vf[2][C::DT];
-                auto read_v_group = [&](int c, bf16x8 (&dst)[C::DT]) {
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt) {
-                        const unsigned char* p = Vt + v_roff[dt] + c * 16 * C::ROW;   // rows 16c + ...
-                        const bf16x4 lo = ds_read_tr16(p);
-                        const bf16x4 hi = ds_read_tr16(p + 8 * C::ROW);
-                        dst[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    }
-                };
-                read_v_group(0, vf[0]);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     if (c + 1 < 4) read_v_group(c + 1, vf[(c + 1) & 1]);
