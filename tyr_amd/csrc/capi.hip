@@ -18,12 +18,14 @@ inline bool fits_int(uint64_t v) { return v <= (uint64_t)INT_MAX; }
 constexpr uint64_t kMaxSplits = 64;
 
 uint64_t auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {
-    // Aim for about 4 workgroups (16 waves) per CU on 256 CUs with at least 256 kv rows per
-    // workgroup, so that every wave has a few 32-row steps to pipeline.
+    // One workgroup (8 waves) per (batch, kv head) already fills the 256 CUs when there are at
+    // least 256 such groups: then a single split is best (no partials, no second pass).  With
+    // fewer groups the KV length is cut so that about 256 workgroups exist, as long as every wave
+    // keeps at least two 32-row steps.
     const uint64_t groups = B * Hkv;
     if (groups == 0) return 1;
-    uint64_t s = (1024 + groups - 1) / groups;
-    const uint64_t max_by_len = L / 256 ? L / 256 : 1;
+    uint64_t s = (256 + groups - 1) / groups;
+    const uint64_t max_by_len = L / 512 ? L / 512 : 1;
     if (s > max_by_len) s = max_by_len;
     if (s < 1) s = 1;
     if (s > kMaxSplits) s = kMaxSplits;

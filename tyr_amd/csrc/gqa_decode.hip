@@ -9,7 +9,7 @@
 // partial results are merged with the online-softmax algebra
 //   m = max m_s ; l = sum l_s 2^(m_s-m) ; O = sum O_s 2^(m_s-m) / l ; LSE = ln l + m ln 2.
 //
-// First pass.  grid = (splits, B*Hkv), 4 waves per workgroup; each wave walks its own slice of
+// First pass.  grid = (splits, B*Hkv), 8 waves per workgroup; each wave walks its own slice of
 // the split in steps of 32 kv rows with the 16x16x32 bf16 MFMA:
 //   S^T (16 kv x 16 q)  = K rows (row operand: lane l holds row l%16, 8 d at 32i + 8(l/16))
 //                         x Q^T (column operand, zero beyond the G = Hq/Hkv real heads)
@@ -18,14 +18,15 @@
 // 8x..8x+7 of 8 rows), transposed 8x8 in registers, and product j then covers d = 8x + j.
 // The 8 rows a lane group takes are exactly the kv rows whose probabilities the S^T accumulator
 // layout leaves in that lane group, so P^T needs no cross-lane movement.
-// The 4 waves merge through LDS and the workgroup writes one f32 partial (O, m, l) per split.
+// The waves merge through LDS and the workgroup writes one f32 partial (O, m, l) per split -- or,
+// when there is a single split, the final bf16 O and LSE (no second pass).
 #include "common.hpp"
 #include "launch.hpp"
 
 namespace tyr {
 
 namespace dec {
-constexpr int THREADS = 256, WAVES = 4, STEP = 32, D = 128, QPAD = 16;
+constexpr int STEP = 32, D = 128, QPAD = 16;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
@@ -35,11 +36,16 @@ struct Buf {
 };
 }  // namespace dec
 
-__global__ __launch_bounds__(dec::THREADS) void gqa_decode_split_kernel(
+// WAVES waves per workgroup share one split.  With a single split (S == 1) the workgroup writes
+// the final bf16 O and LSE itself and the second pass is skipped.
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     float* __restrict__ part_o, float* __restrict__ part_m, float* __restrict__ part_l,
+    uint16_t* __restrict__ O, float* __restrict__ LSE,
     int Hq, int Hkv, int G, int L, long kv_stride, int S, int chunk, int wchunk, float scale_log2) {
     using namespace dec;
+    constexpr int THREADS = 64 * WAVES;
     extern __shared__ __attribute__((aligned(16))) float smem[];   // [WAVES][G][D] O, then [WAVES][QPAD] m, l
 
     const int t = threadIdx.x;
@@ -155,7 +161,7 @@ __global__ __launch_bounds__(dec::THREADS) void gqa_decode_split_kernel(
         }
     }
 
-    // ---- merge the 4 waves through LDS.  oacc[j][rr] is O^T[d = 32g + 8rr + j][q = x].
+    // ---- merge the waves through LDS.  oacc[j][rr] is O^T[d = 32g + 8rr + j][q = x].
     float* so = smem;                              // [WAVES][G][D]
     float* sm = smem + WAVES * G * D;              // [WAVES][QPAD]
     float* sl = sm + WAVES * QPAD;                 // [WAVES][QPAD]
@@ -185,9 +191,15 @@ __global__ __launch_bounds__(dec::THREADS) void gqa_decode_split_kernel(
                 l += sl[ww * QPAD + qh] * wgt;
             }
         }
-        const size_t ph = ((size_t)b * Hq + (size_t)kvh * G + qh) * S + split;
-        part_o[ph * D + d] = o;
-        if (d == 0) { part_m[ph] = m; part_l[ph] = l; }
+        const size_t head = (size_t)b * Hq + (size_t)kvh * G + qh;
+        if (S == 1) {
+            O[head * D + d] = (uint16_t)(pack_bf16(o / l, 0.0f) & 0xffffu);
+            if (d == 0 && LSE != nullptr) LSE[head] = logf(l) + m * LN2;
+        } else {
+            const size_t ph = head * S + split;
+            part_o[ph * D + d] = o;
+            if (d == 0) { part_m[ph] = m; part_l[ph] = l; }
+        }
     }
 }
 
@@ -223,6 +235,7 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
                       void* workspace, hipStream_t stream) {
     using namespace dec;
     (void)D;
+    constexpr int WAVES = 8;
     const int G = Hq / Hkv;
     const int S = num_splits;
     int chunk = (L + S - 1) / S;
@@ -235,15 +248,23 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
     float* part_l = part_m + (size_t)B * Hq * S;
 
     const size_t lds = (size_t)(WAVES * G * dec::D + 2 * WAVES * QPAD) * sizeof(float);
-    dim3 grid((unsigned)S, (unsigned)(B * Hkv)), block(THREADS);
-    hipLaunchKernelGGL(gqa_decode_split_kernel, grid, block, lds, stream,
+    dim3 grid((unsigned)S, (unsigned)(B * Hkv)), block(64 * WAVES);
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&gqa_decode_split_kernel<WAVES>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (WAVES * QPAD * dec::D + 2 * WAVES * QPAD) * (int)sizeof(float));
+    if (attr != hipSuccess) return -1;
+    hipLaunchKernelGGL(gqa_decode_split_kernel<WAVES>, grid, block, lds, stream,
                        static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k),
-                       static_cast<const uint16_t*>(v), part_o, part_m, part_l, Hq, Hkv, G, L,
-                       (long)kv_stride, S, chunk, wchunk, scale * LOG2E);
+                       static_cast<const uint16_t*>(v), part_o, part_m, part_l,
+                       static_cast<uint16_t*>(o), lse, Hq, Hkv, G, L, (long)kv_stride, S, chunk, wchunk,
+                       scale * LOG2E);
     if (hipGetLastError() != hipSuccess) return -1;
-    hipLaunchKernelGGL(gqa_decode_combine_kernel, dim3((unsigned)(B * Hq)), dim3(dec::D), 0, stream,
-                       part_o, part_m, part_l, static_cast<uint16_t*>(o), lse, S);
-    return hipGetLastError() == hipSuccess ? 0 : -1;
+    if (S > 1) {
+        hipLaunchKernelGGL(gqa_decode_combine_kernel, dim3((unsigned)(B * Hq)), dim3(dec::D), 0, stream,
+                           part_o, part_m, part_l, static_cast<uint16_t*>(o), lse, S);
+        if (hipGetLastError() != hipSuccess) return -1;
+    }
+    return 0;
 }
 
 }  // namespace tyr
