@@ -180,6 +180,172 @@ __global__ __launch_bounds__(gemm::THREADS) void gemm_bf16_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Fast path for M % 256 == 0, N % 256 == 0, K % 64 == 0.
+//
+// Same 256x256x64 decomposition, but the slices travel from global memory straight into LDS
+// (no register staging, no LDS stores from the ALU), rows are unpadded with XOR-swizzled 16-byte
+// chunks, and when B is [K,N] it stays row-major in LDS: its MFMA fragments (8 consecutive k for
+// one n) are gathered by the transposing LDS read.  Fragments for k-step s+1 are requested before
+// the 16 MFMAs of k-step s are issued.
+namespace gemm2 {
+constexpr int BM = 256, BN = 256, BK = 64, THREADS = 256;
+constexpr int A_TILE = BM * BK * 2;                  // 32 KiB: [256 m][8 chunks]
+constexpr int B_TILE = BN * BK * 2;                  // 32 KiB: [64 k][32 chunks] or [256 n][8 chunks]
+constexpr int STAGE = A_TILE + B_TILE;
+constexpr int LDS_BYTES = 2 * STAGE;                 // 128 KiB
+constexpr int GROUP_M = 4;
+}  // namespace gemm2
+
+template <bool TRANS_B>
+__global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, int tiles_m, int tiles_n) {
+    using namespace gemm2;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = w >> 1, wn = w & 1;
+
+    const uint32_t nblk = (uint32_t)tiles_m * (uint32_t)tiles_n;
+    const uint32_t pid = xcd_remap(blockIdx.x, nblk);
+    const uint32_t per_group = GROUP_M * (uint32_t)tiles_n;
+    const uint32_t grp = pid / per_group;
+    const uint32_t first_m = grp * GROUP_M;
+    const uint32_t gsz = min((uint32_t)tiles_m - first_m, (uint32_t)GROUP_M);
+    const int tm = (int)(first_m + (pid % per_group) % gsz);
+    const int tn = (int)((pid % per_group) / gsz);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- global -> LDS requests.  Each wave owns a quarter of each tile: 8 instructions of 1 KiB.
+    // A (and B when TRANS_B): 8 rows of 128 B per instruction; chunk c of row m is stored at
+    // position c ^ (m & 7).  B when !TRANS_B: 2 rows of 512 B per instruction; chunk c of row k is
+    // stored at position c ^ ((k & 3) << 2).
+    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K * 2, (size_t)0xffffffffu));
+    const u32x4 b_rsrc = TRANS_B
+        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K * 2, (size_t)0xffffffffu))
+        : make_raw_rsrc(B + n0, (uint32_t)min(((size_t)K * N - n0) * 2, (size_t)0xffffffffu));
+    int a_voff[8], b_voff[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        const int row = (w * 8 + m) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ (row & 7);
+        a_voff[m] = row * K * 2 + c * 16;
+        if (TRANS_B) {
+            b_voff[m] = row * K * 2 + c * 16;
+        } else {
+            const int krow = (w * 8 + m) * 2 + (lane >> 5);
+            const int cb = (lane & 31) ^ ((krow & 3) << 2);
+            b_voff[m] = krow * N * 2 + cb * 16;
+        }
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
+    // quarter q (0..3) of the requests for slice kt into stage st: 2 A + 2 B instructions
+    auto issue_quarter = [&](int st, int kt, int q) {
+        const int a_soff = kt * BK * 2;
+        const int b_soff = TRANS_B ? kt * BK * 2 : kt * BK * N * 2;
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
+#pragma unroll
+        for (int m = 2 * q; m < 2 * q + 2; ++m) {
+            load_global_to_lds_16(a_rsrc, dst + m * 1024, a_voff[m], a_soff);
+            load_global_to_lds_16(b_rsrc, dst + A_TILE + m * 1024, b_voff[m], b_soff);
+        }
+    };
+
+    // ---- fragment addresses
+    // A fragment (m tile i, k-step s): row wm*128 + 32i + r, chunk (2s + g) ^ (r & 7).
+    int a_roff[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) a_roff[s] = (wm * 128 + r) * 128 + (((2 * s + g) ^ (r & 7)) * 16);
+    // B fragment, TRANS_B: like A with n rows.  Otherwise (row-major [k][n]) via the transposing
+    // read: as a source lane this lane points at k row 8(b/2) + 4h + j (j = (lane%16)/4) of the
+    // k-step, 8 bytes at n = wn*128 + 32jt + 16(b&1) + 4(lane%4); jt enters through the swizzle.
+    int b_roff[4];
+    if (TRANS_B) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) b_roff[s] = A_TILE + (wn * 128 + r) * 128 + (((2 * s + g) ^ (r & 7)) * 16);
+    } else {
+        const int i16 = lane & 15, b16 = lane >> 4;
+        const int js = i16 >> 2, qs = i16 & 3;
+        const int krow = 8 * (b16 >> 1) + js;
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) {
+            const int c = wn * 16 + 4 * jt + 2 * (b16 & 1) + (qs >> 1);
+            b_roff[jt] = A_TILE + krow * 512 + ((c ^ (js << 2)) * 16) + (qs & 1) * 8;
+        }
+    }
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    auto read_frags = [&](const unsigned char* St, int s, bf16x8 (&af)[4], bf16x8 (&bf)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(St + a_roff[s] + i * 32 * 128);
+        if (TRANS_B) {
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) bf[jt] = *reinterpret_cast<const bf16x8*>(St + b_roff[s] + jt * 32 * 128);
+        } else {
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const unsigned char* p = St + b_roff[jt] + s * 16 * 512;
+                const bf16x4 lo = ds_read_tr16(p);
+                const bf16x4 hi = ds_read_tr16(p + 4 * 512);
+                bf[jt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+    };
+
+    const int KT = K / BK;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) issue_quarter(0, 0, q);
+    wait_vmcnt0();
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int st = kt & 1;
+        const unsigned char* St = lds + st * STAGE;
+        const bool more = kt + 1 < KT;
+        bf16x8 af[2][4], bf[2][4];
+        read_frags(St, 0, af[0], bf[0]);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            if (more) issue_quarter(st ^ 1, kt + 1, s);
+            if (s + 1 < 4) read_frags(St, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[s & 1][j], af[s & 1][i], acc[i][j]);
+        }
+        wait_vmcnt0();
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds m = ..+r and, per register quad q4, n = ..+8*q4+4*g+[0,4)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint16_t* crow = C + (size_t)(m0 + wm * 128 + i * 32 + r) * N;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int gn = n0 + wn * 128 + j * 32 + q4 * 8 + g * 4;
+                u32x2 v;
+                v.x = pack_bf16(acc[i][j][q4 * 4 + 0], acc[i][j][q4 * 4 + 1]);
+                v.y = pack_bf16(acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
+                st_global_8(crow + gn, v);
+            }
+        }
+    }
+}
+
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
                      hipStream_t stream) {
     using namespace gemm;
@@ -189,6 +355,23 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
     auto A = static_cast<const uint16_t*>(a);
     auto Bp = static_cast<const uint16_t*>(b);
     auto Cp = static_cast<uint16_t*>(c);
+    // 32-bit buffer offsets: one 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
+    const bool fast_ok = !edge && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
+                         (trans_b || (size_t)K * N * 2 < ((size_t)1 << 32));
+    if (fast_ok) {
+#define TYR_GEMM_FAST(TB)                                                                         \
+        do {                                                                                      \
+            static const hipError_t attr = hipFuncSetAttribute(                                   \
+                reinterpret_cast<const void*>(&gemm_bf16_fast_kernel<TB>),                        \
+                hipFuncAttributeMaxDynamicSharedMemorySize, gemm2::LDS_BYTES);                    \
+            if (attr != hipSuccess) return -1;                                                    \
+            hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB>), grid, block, gemm2::LDS_BYTES, stream, \
+                               A, Bp, Cp, M, N, K, tiles_m, tiles_n);                             \
+        } while (0)
+        if (trans_b) TYR_GEMM_FAST(true); else TYR_GEMM_FAST(false);
+#undef TYR_GEMM_FAST
+        return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
 #define TYR_GEMM_LAUNCH(TB, ED)                                                                   \
     do {                                                                                          \
         static const hipError_t attr = hipFuncSetAttribute(                                       \
