@@ -309,23 +309,33 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     wait_vmcnt0();
     __syncthreads();
 
+    // Steady state per slice: the next slice is requested during k-steps 0 and 1; fragments for
+    // k-step s+1 are read before the MFMAs of k-step s; before the MFMAs of the last k-step the
+    // workgroup synchronises and already reads the first fragments of the next slice, so the
+    // barrier and the LDS latency hide under 16 MFMAs.  (Past the last slice the requests and
+    // reads touch the idle stage / stale data and are never used.)
+    bf16x8 af[2][4], bf[2][4];
+    read_frags(lds, 0, af[0], bf[0]);
     for (int kt = 0; kt < KT; ++kt) {
         const int st = kt & 1;
         const unsigned char* St = lds + st * STAGE;
-        const bool more = kt + 1 < KT;
-        bf16x8 af[2][4], bf[2][4];
-        read_frags(St, 0, af[0], bf[0]);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            if (more) issue_quarter(st ^ 1, kt + 1, s);
-            if (s + 1 < 4) read_frags(St, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            if (s < 2) { issue_quarter(st ^ 1, kt + 1, 2 * s); issue_quarter(st ^ 1, kt + 1, 2 * s + 1); }
+            if (s < 3) {
+                read_frags(St, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            } else {
+                wait_vmcnt0();
+                __syncthreads();
+                read_frags(lds + (st ^ 1) * STAGE, 0, af[0], bf[0]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[s & 1][j], af[s & 1][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        wait_vmcnt0();
-        __syncthreads();
     }
 
     // ---- epilogue: lane holds m = ..+r and, per register quad q4, n = ..+8*q4+4*g+[0,4)
