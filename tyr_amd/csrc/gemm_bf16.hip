@@ -221,7 +221,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 
     // ---- global -> LDS requests.  Each wave owns a quarter of each tile: 8 instructions of 1 KiB.
     // A (and B when TRANS_B): 8 rows of 128 B per instruction; chunk c of row m is stored at
-    // position c ^ (m & 7).  B when !TRANS_B: 2 rows of 512 B per instruction; chunk c of row k is
+    // position c ^ ((m >> 1) & 7), so 16 consecutive rows put one logical chunk on all 64 banks.  B when !TRANS_B: 2 rows of 512 B per instruction; chunk c of row k is
     // stored at position c ^ ((k & 3) << 2).
     const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K * 2, (size_t)0xffffffffu));
     const u32x4 b_rsrc = TRANS_B
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
         const int row = (w * 8 + m) * 8 + (lane >> 3);
-        const int c = (lane & 7) ^ (row & 7);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
         a_voff[m] = row * K * 2 + c * 16;
         if (TRANS_B) {
             b_voff[m] = row * K * 2 + c * 16;
@@ -256,17 +256,17 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     };
 
     // ---- fragment addresses
-    // A fragment (m tile i, k-step s): row wm*128 + 32i + r, chunk (2s + g) ^ (r & 7).
+    // A fragment (m tile i, k-step s): row wm*128 + 32i + r, chunk (2s + g) ^ ((r >> 1) & 7).
     int a_roff[4];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) a_roff[s] = (wm * 128 + r) * 128 + (((2 * s + g) ^ (r & 7)) * 16);
+    for (int s = 0; s < 4; ++s) a_roff[s] = (wm * 128 + r) * 128 + (((2 * s + g) ^ ((r >> 1) & 7)) * 16);
     // B fragment, TRANS_B: like A with n rows.  Otherwise (row-major [k][n]) via the transposing
     // read: as a source lane this lane points at k row 8(b/2) + 4h + j (j = (lane%16)/4) of the
     // k-step, 8 bytes at n = wn*128 + 32jt + 16(b&1) + 4(lane%4); jt enters through the swizzle.
     int b_roff[4];
     if (TRANS_B) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) b_roff[s] = A_TILE + (wn * 128 + r) * 128 + (((2 * s + g) ^ (r & 7)) * 16);
+        for (int s = 0; s < 4; ++s) b_roff[s] = A_TILE + (wn * 128 + r) * 128 + (((2 * s + g) ^ ((r >> 1) & 7)) * 16);
     } else {
         const int i16 = lane & 15, b16 = lane >> 4;
         const int js = i16 >> 2, qs = i16 & 3;
