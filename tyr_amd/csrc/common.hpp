@@ -138,6 +138,34 @@ __device__ __forceinline__ bf16x4 ds_read_tr16(const void* lds_ptr) {
     return __builtin_bit_cast(bf16x4, v);
 }
 
+// Epilogue of the 256x256-tile GEMMs: one wave's 128x128 f32 accumulator quadrant (4x4 MFMA tiles
+// computed with the B fragment as row operand: lane = m row l%32, register e <-> n = 8(e/4) +
+// 4(l/32) + e%4) goes to global memory as bf16 rows.  Each 32-row band passes through a private
+// LDS scratch (32 rows x 272 B) so that the global stores are 16 bytes per lane along rows.
+constexpr int kEpilogueScratchBytes = 32 * 272;
+__device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], float scale, unsigned char* scratch,
+                                                    uint16_t* c_quadrant, int ldc, int lane) {
+    const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                u32x2 v;
+                v.x = pack_bf16(acc[i][j][q4 * 4 + 0] * scale, acc[i][j][q4 * 4 + 1] * scale);
+                v.y = pack_bf16(acc[i][j][q4 * 4 + 2] * scale, acc[i][j][q4 * 4 + 3] * scale);
+                *reinterpret_cast<u32x2*>(scratch + r * 272 + (j * 32 + q4 * 8 + g * 4) * 2) = v;
+            }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int row = (lane >> 4) + 4 * k;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * 272 + (lane & 15) * 16);
+            st_global_16(c_quadrant + (size_t)(i * 32 + row) * ldc + (lane & 15) * 8, v);
+        }
+    }
+}
+
 // Grid remap for the 8 XCDs of an MI355X: consecutive workgroup ids are dealt round-robin
 // to the XCDs, each with its own L2.  This returns a logical id such that the workgroups
 // that land on one XCD cover one contiguous range of logical ids (so neighbours in the

@@ -338,22 +338,9 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         }
     }
 
-    // ---- epilogue: lane holds m = ..+r and, per register quad q4, n = ..+8*q4+4*g+[0,4)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint16_t* crow = C + (size_t)(m0 + wm * 128 + i * 32 + r) * N;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int gn = n0 + wn * 128 + j * 32 + q4 * 8 + g * 4;
-                u32x2 v;
-                v.x = pack_bf16(acc[i][j][q4 * 4 + 0], acc[i][j][q4 * 4 + 1]);
-                v.y = pack_bf16(acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
-                st_global_8(crow + gn, v);
-            }
-        }
-    }
+    // ---- epilogue (all requests have landed and every wave is past its last fragment read)
+    store_quadrant_bf16(acc, 1.0f, lds + w * kEpilogueScratchBytes,
+                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane);
 }
 
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
