@@ -105,6 +105,14 @@ __device__ __forceinline__ void pin_registers(bf16x8& v) {
     v = __builtin_bit_cast(bf16x8, u);
 }
 
+// ds_read_b64_tr_b8: transposing LDS read for bytes.  Within each block of 16 lanes, lane 8q+p
+// receives byte p of the 8-byte pieces addressed by lanes q, q+2, q+4, ..., q+14 of the block.
+__device__ __forceinline__ u32x2 ds_read_tr8(const void* lds_ptr) {
+    typedef __attribute__((ext_vector_type(2))) int i32x2;
+    const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(lds_ptr));
+    return __builtin_bit_cast(u32x2, v);
+}
+
 // Buffer resource (V#) for raw byte-addressed access to [base, base + bytes): loads beyond the
 // range return zero.
 __device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, uint32_t bytes) {

@@ -197,6 +197,175 @@ __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Fast path for M % 256 == 0, N % 256 == 0, K % 128 == 0: slices go from global memory straight
+// into LDS, unpadded rows with XOR-swizzled 16-byte chunks; a [K,N] B stays row-major in LDS and
+// its fragments (32 consecutive k for one n) are gathered with the byte-transposing LDS read.
+namespace gemm8f {
+constexpr int BM = 256, BN = 256, BK = 128, THREADS = 256;
+constexpr int A_TILE = BM * BK;                      // 32 KiB: [256 m][8 chunks]
+constexpr int B_TILE = BN * BK;                      // 32 KiB: [128 k][16 chunks] or [256 n][8 chunks]
+constexpr int STAGE = A_TILE + B_TILE;
+constexpr int LDS_BYTES = 2 * STAGE;
+constexpr int GROUP_M = 4;
+}  // namespace gemm8f
+
+template <bool TRANS_B>
+__global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, int tiles_m, int tiles_n, float scale) {
+    using namespace gemm8f;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = w >> 1, wn = w & 1;
+
+    const uint32_t nblk = (uint32_t)tiles_m * (uint32_t)tiles_n;
+    const uint32_t pid = xcd_remap(blockIdx.x, nblk);
+    const uint32_t per_group = GROUP_M * (uint32_t)tiles_n;
+    const uint32_t grp = pid / per_group;
+    const uint32_t first_m = grp * GROUP_M;
+    const uint32_t gsz = min((uint32_t)tiles_m - first_m, (uint32_t)GROUP_M);
+    const int tm = (int)(first_m + (pid % per_group) % gsz);
+    const int tn = (int)((pid % per_group) / gsz);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- global -> LDS requests (8 instructions of 1 KiB per wave and tile).
+    // A (and B when TRANS_B): 8 rows of 128 B per instruction, chunk c of row m at c ^ ((m>>1)&7).
+    // B when !TRANS_B: 4 rows of 256 B per instruction, chunk c of row k at c ^ ((k&7)<<1).
+    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K, (size_t)0xffffffffu));
+    const u32x4 b_rsrc = TRANS_B
+        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K, (size_t)0xffffffffu))
+        : make_raw_rsrc(B + n0, (uint32_t)min((size_t)K * N - n0, (size_t)0xffffffffu));
+    int a_voff[8], b_voff[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        const int row = (w * 8 + m) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        a_voff[m] = row * K + c * 16;
+        if (TRANS_B) {
+            b_voff[m] = row * K + c * 16;
+        } else {
+            const int krow = (w * 8 + m) * 4 + (lane >> 4);
+            const int cb = (lane & 15) ^ ((krow & 7) << 1);
+            b_voff[m] = krow * N + cb * 16;
+        }
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
+    auto issue_half = [&](int st, int kt, int h) {
+        const int a_soff = kt * BK;
+        const int b_soff = TRANS_B ? kt * BK : kt * BK * N;
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
+#pragma unroll
+        for (int m = 4 * h; m < 4 * h + 4; ++m) {
+            load_global_to_lds_16(a_rsrc, dst + m * 1024, a_voff[m], a_soff);
+            load_global_to_lds_16(b_rsrc, dst + A_TILE + m * 1024, b_voff[m], b_soff);
+        }
+    };
+
+    // ---- fragment addresses.  k-step s covers bytes [64s, 64s+64) of a row; lane group g takes
+    // the 32 bytes at 64s + 32g, i.e. chunks 4s + 2g and 4s + 2g + 1.
+    int a_roff[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            a_roff[s][h] = (wm * 128 + r) * 128 + (((4 * s + 2 * g + h) ^ ((r >> 1) & 7)) * 16);
+    int b_roff[4];    // TRANS_B: [s][h] like A.  Otherwise [jt]: source-lane address for n tile jt.
+    if (TRANS_B) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                b_roff[2 * s + h] = A_TILE + (wn * 128 + r) * 128 + (((4 * s + 2 * g + h) ^ ((r >> 1) & 7)) * 16);
+    } else {
+        // As a source lane of the byte-transposing read: k row 32(b/2) + (lane%16)/2 (+64s + 8h),
+        // 8 bytes at n = wn*128 + 32jt + 16(b&1) + 8(lane%2).
+        const int i16 = lane & 15, b16 = lane >> 4;
+        const int js = i16 >> 1, qs = i16 & 1;
+        const int krow = 32 * (b16 >> 1) + js;
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) {
+            const int c = wn * 8 + 2 * jt + (b16 & 1);
+            b_roff[jt] = A_TILE + krow * 256 + ((c ^ (js << 1)) * 16) + qs * 8;
+        }
+    }
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    auto read_frags = [&](const unsigned char* St, int s, i32x8 (&af)[4], i32x8 (&bf)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + a_roff[s][0] + i * 32 * 128);
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + a_roff[s][1] + i * 32 * 128);
+            af[i] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        }
+        if (TRANS_B) {
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s] + jt * 32 * 128);
+                const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s + 1] + jt * 32 * 128);
+                bf[jt] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+            }
+        } else {
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const unsigned char* p = St + b_roff[jt] + s * 64 * 256;
+                const u32x2 y0 = ds_read_tr8(p);
+                const u32x2 y1 = ds_read_tr8(p + 8 * 256);
+                const u32x2 y2 = ds_read_tr8(p + 16 * 256);
+                const u32x2 y3 = ds_read_tr8(p + 24 * 256);
+                bf[jt] = i32x8{(int)y0.x, (int)y0.y, (int)y1.x, (int)y1.y, (int)y2.x, (int)y2.y, (int)y3.x, (int)y3.y};
+            }
+        }
+    };
+
+    const int KT = K / BK;
+    issue_half(0, 0, 0);
+    issue_half(0, 0, 1);
+    wait_vmcnt0();
+    __syncthreads();
+
+    // Per slice: k-step 0 requests the next slice and reads the fragments of k-step 1; before the
+    // MFMAs of k-step 1 the workgroup synchronises and reads the first fragments of the next slice.
+    i32x8 af[2][4], bf[2][4];
+    read_frags(lds, 0, af[0], bf[0]);
+    for (int kt = 0; kt < KT; ++kt) {
+        const int st = kt & 1;
+        const unsigned char* St = lds + st * STAGE;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (s == 0) {
+                issue_half(st ^ 1, kt + 1, 0);
+                issue_half(st ^ 1, kt + 1, 1);
+                read_frags(St, 1, af[1], bf[1]);
+            } else {
+                wait_vmcnt0();
+                __syncthreads();
+                read_frags(lds + (st ^ 1) * STAGE, 0, af[0], bf[0]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    store_quadrant_bf16(acc, scale, lds + w * kEpilogueScratchBytes,
+                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane);
+}
+
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
                     int trans_b, hipStream_t stream) {
     using namespace gemm8;
@@ -206,6 +375,23 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
     auto A = static_cast<const uint8_t*>(aq);
     auto Bp = static_cast<const uint8_t*>(bq);
     auto Cp = static_cast<uint16_t*>(c);
+    // 32-bit buffer offsets: a 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
+    const bool fast_ok = !edge && (size_t)256 * K < ((size_t)1 << 31) &&
+                         (trans_b || (size_t)K * N < ((size_t)1 << 32));
+    if (fast_ok) {
+#define TYR_GEMM8_FAST(TB)                                                                        \
+        do {                                                                                      \
+            static const hipError_t attr = hipFuncSetAttribute(                                   \
+                reinterpret_cast<const void*>(&gemm_fp8_fast_kernel<TB>),                         \
+                hipFuncAttributeMaxDynamicSharedMemorySize, gemm8f::LDS_BYTES);                   \
+            if (attr != hipSuccess) return -1;                                                    \
+            hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB>), grid, block, gemm8f::LDS_BYTES, stream, \
+                               A, Bp, Cp, M, N, K, tiles_m, tiles_n, scale);                      \
+        } while (0)
+        if (trans_b) TYR_GEMM8_FAST(true); else TYR_GEMM8_FAST(false);
+#undef TYR_GEMM8_FAST
+        return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
 #define TYR_GEMM8_LAUNCH(TB, ED)                                                                  \
     do {                                                                                          \
         static const hipError_t attr = hipFuncSetAttribute(                                       \
