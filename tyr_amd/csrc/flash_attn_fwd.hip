@@ -322,11 +322,14 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         if (j + 1 < nkv) tile_step(sB, sA, j + 1);
     }
 
-    // ---- finalize: O /= l, LSE = ln l + m
+    // ---- finalize: O /= l, LSE = ln l + m.  The wave's 32 x D block of O goes through a private LDS
+    // scratch (all K/V stages are dead after the last barrier) so that global stores are 16 bytes
+    // per lane along rows.
     const float ltot = sum_xor32(lsum);
     const float inv = 1.0f / ltot;
-    if (qpos < N) {
-        uint16_t* orow = O + head_off + (size_t)qpos * D;
+    {
+        constexpr int SROW = D * 2 + 16;
+        unsigned char* scratch = lds + w * (32 * SROW);
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
 #pragma unroll
@@ -334,11 +337,19 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                 u32x2 v;
                 v.x = pack_bf16(oacc[dt][4 * q4 + 0] * inv, oacc[dt][4 * q4 + 1] * inv);
                 v.y = pack_bf16(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv);
-                st_global_8(orow + dt * 32 + q4 * 8 + g * 4, v);
+                *reinterpret_cast<u32x2*>(scratch + r * SROW + (dt * 32 + q4 * 8 + g * 4) * 2) = v;
             }
         }
-        if (LSE != nullptr && g == 0) LSE[(size_t)bh * N + qpos] = logf(ltot) + m2 * LN2;
+        constexpr int CH = D / 8;                   // 16-byte chunks per row
+        constexpr int RPI = 64 / CH;                // rows per store instruction
+#pragma unroll
+        for (int k = 0; k < 32 / RPI; ++k) {
+            const int row = lane / CH + RPI * k;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * SROW + (lane % CH) * 16);
+            if (qw0 + row < N) st_global_16(O + head_off + (size_t)(qw0 + row) * D + (lane % CH) * 8, v);
+        }
     }
+    if (qpos < N && LSE != nullptr && g == 0) LSE[(size_t)bh * N + qpos] = logf(ltot) + m2 * LN2;
 }
 
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
