@@ -32,6 +32,13 @@ if ROOT not in sys.path:
 
 PEAK = {"mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "hbm": 8000.0}   # TFLOP/s, TFLOP/s, GB/s
 
+# HBM bytes per launch of the dominant kernel, measured with `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` on this same script (one counter per run) and scaled by what the same counters
+# read for the 1 GiB copy of --workload copy_1gib (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the raw
+# figures are kept as text under profiles/.
+TRAFFIC = {"attn_fwd_causal": 815_316_992 + 272_629_760, "gqa_decode": 1_074_495_488 + 270_336,
+           "gemm_bf16": 202_589_594 + 33_554_432, "gemm_fp8": 810_477_568 + 136_314_880}
+
 
 def _events(torch, n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -70,7 +77,8 @@ def wl_attn(torch, tyr, steps, warmup, cpu):
         "config": {"workload": "causal flash-attention forward, bf16, B=16 H=16 N=4096 D=128, O + LSE",
                    "flop_convention": "4*B*H*N^2*D/2 (causal half)", "scale": "1/sqrt(128)"},
         "roofline": {"bound": "mfma", "kernel": "flash_attn_fwd_kernel<128,true>", "achieved": tf,
-                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"], "traffic": None},
+                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"],
+                     "traffic": TRAFFIC["attn_fwd_causal"]},
     }
     if cpu:
         from oracle import libtorch_path as lt
@@ -113,9 +121,9 @@ def wl_decode(torch, tyr, steps, warmup, cpu):
                    "bytes_convention": "K + V + Q + O = 1,074,266,112 B (split partials excluded)",
                    "num_splits": int(__import__("tyr_amd._lib", fromlist=["load"]).load()
                                      .tyr_hip_gqa_decode_auto_splits(B, Hkv, L)),
-                   "note": "time covers both passes (split kernel + combine kernel)"},
-        "roofline": {"bound": "hbm", "kernel": "gqa_decode_split_kernel (+combine)", "achieved": gbs,
-                     "peak": PEAK["hbm"], "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": None},
+                   "note": "one split per (batch, kv head) at this shape: the first pass writes O and LSE itself"},
+        "roofline": {"bound": "hbm", "kernel": "gqa_decode_split_kernel<8>", "achieved": gbs,
+                     "peak": PEAK["hbm"], "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": TRAFFIC["gqa_decode"]},
     }
     if cpu:
         from oracle import libtorch_path as lt
@@ -148,8 +156,9 @@ def wl_gemm_bf16(torch, tyr, steps, warmup, cpu):
         "dtype": "bf16",
         "config": {"workload": "bf16 GEMM M=N=K=4096, row-major A and B, f32 accumulate, bf16 out",
                    "input_std": "K^-1/4 = 0.125"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel<false,false>", "achieved": tf,
-                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"], "traffic": None},
+        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_fast_kernel<false>", "achieved": tf,
+                     "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"],
+                     "traffic": TRAFFIC["gemm_bf16"]},
     }
     if cpu:
         from oracle import libtorch_path as lt
@@ -178,8 +187,9 @@ def wl_gemm_fp8(torch, tyr, steps, warmup, cpu):
         "metric": "GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
         "dtype": "fp8_e4m3",
         "config": {"workload": "fp8 e4m3 GEMM M=N=K=8192, per-tensor f32 scales, bf16 out"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_fp8_kernel<false,false>", "achieved": tf,
-                     "peak": PEAK["mfma_fp8"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_fp8"], "traffic": None},
+        "roofline": {"bound": "mfma", "kernel": "gemm_fp8_fast_kernel<false>", "achieved": tf,
+                     "peak": PEAK["mfma_fp8"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_fp8"],
+                     "traffic": TRAFFIC["gemm_fp8"]},
     }
     if cpu:
         from oracle import libtorch_path as lt
