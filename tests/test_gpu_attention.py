@@ -46,6 +46,34 @@ def test_flash_attn_matches_oracle(gpu, B, H, N, D, causal):
     assert max_abs(lse.cpu(), lset) <= 1e-3
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_flash_attn_random_shapes(gpu, seed):
+    # randomised e2e in the spirit of the reference's E2E_TRIALS runs: ragged lengths, odd head counts
+    rng = np.random.default_rng(1000 + seed)
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+    N, D = int(rng.integers(1, 1100)), int(rng.choice([64, 128]))
+    causal = bool(rng.integers(0, 2))
+    q, k, v = qkv(500 + seed, B, H, N, D)
+    sc = float(rng.uniform(0.05, 0.2))
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc)
+    o64, lse64 = oracle.attn_fwd_f64(bits(q), bits(k), bits(v), causal, sc)
+    assert max_abs(o.cpu().float(), o64) <= TOL, (B, H, N, D, causal)
+    assert max_abs(lse.cpu(), lse64) <= 1e-3, (B, H, N, D, causal)
+
+
+def test_flash_attn_large_scores_trigger_rescales(gpu):
+    # keys whose scores grow along the sequence force the running maximum to move repeatedly
+    B, H, N, D = 1, 2, 700, 128
+    q, k, v = qkv(31, B, H, N, D)
+    ramp = torch.linspace(0.2, 6.0, N).view(1, 1, N, 1)
+    k = (k.float() * ramp).to(torch.bfloat16)
+    for causal in (False, True):
+        o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal)
+        o64, lse64 = oracle.attn_fwd_f64(bits(q), bits(k), bits(v), causal, 1 / math.sqrt(D))
+        assert max_abs(o.cpu().float(), o64) <= TOL
+        assert max_abs(lse.cpu(), lse64) <= 2e-3
+
+
 def test_flash_attn_causal_closed_forms(gpu):
     B, H, N, D = 1, 2, 300, 128
     q, k, v = qkv(11, B, H, N, D)
@@ -117,6 +145,24 @@ def test_gqa_decode_matches_oracle(gpu, B, Hq, Hkv, L, splits):
     # the LibTorch call sequence of the reference (repeat_interleave + SDPA), fp32
     ref = lt.sdpa_gqa_qkv(q.float(), k.float(), v.float(), False, True)
     assert max_abs(o.cpu().float(), ref) <= TOL
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gqa_decode_random_shapes(gpu, seed):
+    rng = np.random.default_rng(2000 + seed)
+    Hkv = int(rng.integers(1, 5))
+    G = int(rng.choice([1, 2, 4, 7, 16]))
+    B, L = int(rng.integers(1, 4)), int(rng.integers(1, 3000))
+    Lmax = L + int(rng.integers(0, 100))
+    splits = int(rng.choice([0, 1, 2, 5, 16]))
+    D = 128
+    q, = lt.make_inputs(600 + seed, (B, Hkv * G, 1, D))
+    k, v = lt.make_inputs(700 + seed, (B, Hkv, Lmax, D), (B, Hkv, Lmax, D))
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits, kv_len=L)
+    want_o, want_lse = oracle.gqa_decode(bits(q), bits(k), bits(v), sc, max(splits, 1), kv_len=L)
+    assert max_abs(o.cpu().float(), from_bits(want_o).float()) <= TOL, (B, Hkv, G, L, splits)
+    assert max_abs(lse.cpu(), want_lse) <= 1e-3, (B, Hkv, G, L, splits)
 
 
 def test_gqa_decode_split_invariance_and_partial_cache(gpu):

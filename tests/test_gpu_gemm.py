@@ -24,7 +24,7 @@ def gpu():
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 512, 4096), (8, 8, 8),
-                                   (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256)])
+                                   (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256), (768, 512, 320)])
 def test_gemm_bf16_matches_oracle(gpu, M, N, K, trans_b):
     a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
     bb = b.t().contiguous() if trans_b else b
@@ -51,6 +51,24 @@ def test_gemm_bf16_identity_and_permutation_bit_exact(gpu, trans_b):
     assert np.array_equal(bits(got_ap), bits(a[:, torch.argsort(perm)]))
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_gemm_random_shapes(gpu, seed):
+    rng = np.random.default_rng(3000 + seed)
+    M = int(rng.integers(1, 700))
+    N = 16 * int(rng.integers(1, 40))
+    K = 16 * int(rng.integers(1, 60))
+    trans_b = bool(rng.integers(0, 2))
+    a, b = lt.make_inputs(800 + seed, (M, K), (K, N), std=K ** -0.25)
+    bb = b.t().contiguous() if trans_b else b
+    c = gpu.gemm_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
+    assert rel_fro(c, a.float() @ b.float()) <= TOL_FRO, (M, N, K, trans_b)
+    aq, sa = lt.quantize_e4m3(a.float() * 8)
+    bq, sb = lt.quantize_e4m3(b.float() * 8)
+    bqb = bq.t().contiguous() if trans_b else bq
+    c8 = gpu.gemm_fp8(aq.cuda(), bqb.cuda(), sa, sb, trans_b=trans_b).cpu()
+    assert rel_fro(c8, lt.fp8_mm(aq, bq, sa, sb)) <= TOL_FRO, (M, N, K, trans_b)
+
+
 def test_gemm_bf16_full_size_config(gpu):
     # M = N = K = 4096, entries ~ N(0, 1/sqrt(K)) (std K^-1/4), row-major A and B.
     M = N = K = 4096
@@ -75,7 +93,7 @@ def test_gemm_bf16_full_size_config(gpu):
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 256, 384), (16, 16, 16), (300, 272, 80),
-                                   (1, 16, 16), (257, 48, 1040)])
+                                   (1, 16, 16), (257, 48, 1040), (768, 512, 640)])
 def test_gemm_fp8_matches_oracle(gpu, M, N, K, trans_b):
     torch.manual_seed(200 + M + N + K)
     a, b = torch.randn(M, K), torch.randn(K, N)

@@ -94,6 +94,7 @@ int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
     if (!fits_int(N) || !fits_int(B * H) || B * H > (uint64_t)INT_MAX / ((N + 127) / 128))
         return TYR_HIP_ERR_BAD_SHAPE;
+    if (N * D * 2 >= ((uint64_t)1 << 32)) return TYR_HIP_ERR_UNSUPPORTED;   // one head's K or V must stay below 4 GiB
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
     if (lse && (reinterpret_cast<uintptr_t>(lse) & 3u)) return TYR_HIP_ERR_MISALIGNED;
     const int rc = tyr::launch_flash_attn_fwd(q, k, v, o, lse, (int)B, (int)H, (int)N, (int)D,
