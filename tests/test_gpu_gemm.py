@@ -24,7 +24,8 @@ def gpu():
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 512, 4096), (8, 8, 8),
-                                   (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256), (768, 512, 320)])
+                                   (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256), (768, 512, 320),
+                                   (300, 264, 128), (1, 16, 64), (513, 520, 192), (700, 1000, 256)])
 def test_gemm_bf16_matches_oracle(gpu, M, N, K, trans_b):
     a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
     bb = b.t().contiguous() if trans_b else b
@@ -69,6 +70,39 @@ def test_gemm_random_shapes(gpu, seed):
     assert rel_fro(c8, lt.fp8_mm(aq, bq, sa, sb)) <= TOL_FRO, (M, N, K, trans_b)
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("M,N,K", [(300, 264, 128), (257, 8, 64), (1, 272, 256), (511, 504, 72)])
+def test_gemm_ragged_tiles_write_only_c(gpu, M, N, K, trans_b):
+    # C sits inside a larger buffer of a canary value: tiles that overhang M or N must not
+    # write outside the M*N elements of C.
+    from tyr_amd import _lib
+    lib = _lib.load()
+    a, b = lt.make_inputs(4000 + M + N + K, (M, K), (K, N), std=K ** -0.25)
+    bb = b.t().contiguous() if trans_b else b
+    guard = 4096
+    canary = torch.full((guard + M * N + guard,), -7.0, dtype=torch.bfloat16, device="cuda")
+    ad, bd = a.cuda(), bb.cuda()
+    rc = lib.tyr_hip_gemm_bf16(ad.data_ptr(), bd.data_ptr(), canary.data_ptr() + 2 * guard, M, N, K,
+                               int(trans_b), 0)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bool((canary[:guard] == -7.0).all()) and bool((canary[guard + M * N:] == -7.0).all())
+    assert torch.equal(canary[guard:guard + M * N].view(M, N), gpu.gemm_bf16(ad, bd, trans_b=trans_b))
+    if N % 16 == 0 and K % 16 == 0:
+        aq, sa = lt.quantize_e4m3(a.float())
+        bq, sb = lt.quantize_e4m3(b.float())
+        bqb = (bq.t().contiguous() if trans_b else bq).cuda()
+        aqd = aq.cuda()
+        canary.fill_(-7.0)
+        rc = lib.tyr_hip_gemm_fp8(aqd.data_ptr(), bqb.data_ptr(), canary.data_ptr() + 2 * guard, M, N, K,
+                                  float(sa), float(sb), int(trans_b), 0)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert bool((canary[:guard] == -7.0).all()) and bool((canary[guard + M * N:] == -7.0).all())
+        assert torch.equal(canary[guard:guard + M * N].view(M, N),
+                           gpu.gemm_fp8(aqd, bqb, sa, sb, trans_b=trans_b))
+
+
 def test_gemm_bf16_full_size_config(gpu):
     # M = N = K = 4096, entries ~ N(0, 1/sqrt(K)) (std K^-1/4), row-major A and B.
     M = N = K = 4096
@@ -93,7 +127,8 @@ def test_gemm_bf16_full_size_config(gpu):
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 256, 384), (16, 16, 16), (300, 272, 80),
-                                   (1, 16, 16), (257, 48, 1040), (768, 512, 640)])
+                                   (1, 16, 16), (257, 48, 1040), (768, 512, 640),
+                                   (300, 272, 128), (1, 16, 128), (513, 528, 384), (700, 1008, 256)])
 def test_gemm_fp8_matches_oracle(gpu, M, N, K, trans_b):
     torch.manual_seed(200 + M + N + K)
     a, b = torch.randn(M, K), torch.randn(K, N)

@@ -151,8 +151,9 @@ __device__ __forceinline__ bf16x4 ds_read_tr16(const void* lds_ptr) {
 // 4(l/32) + e%4) goes to global memory as bf16 rows.  Each 32-row band passes through a private
 // LDS scratch (32 rows x 272 B) so that the global stores are 16 bytes per lane along rows.
 constexpr int kEpilogueScratchBytes = 32 * 272;
+// rows / cols = how much of the 128x128 quadrant lies inside C (cols a multiple of 8).
 __device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], float scale, unsigned char* scratch,
-                                                    uint16_t* c_quadrant, int ldc, int lane) {
+                                                    uint16_t* c_quadrant, int ldc, int lane, int rows, int cols) {
     const int r = lane & 31, g = lane >> 5;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -169,7 +170,8 @@ __device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], f
         for (int k = 0; k < 8; ++k) {
             const int row = (lane >> 4) + 4 * k;
             const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * 272 + (lane & 15) * 16);
-            st_global_16(c_quadrant + (size_t)(i * 32 + row) * ldc + (lane & 15) * 8, v);
+            if (i * 32 + row < rows && (lane & 15) * 8 < cols)
+                st_global_16(c_quadrant + (size_t)(i * 32 + row) * ldc + (lane & 15) * 8, v);
         }
     }
 }

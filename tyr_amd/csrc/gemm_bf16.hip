@@ -181,7 +181,7 @@ __global__ __launch_bounds__(gemm::THREADS) void gemm_bf16_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path for M % 256 == 0, N % 256 == 0, K % 64 == 0.
+// Fast path for K % 64 == 0 (any M; N % 8 == 0).
 //
 // Same 256x256x64 decomposition, but the slices travel from global memory straight into LDS
 // (no register staging, no LDS stores from the ALU), rows are unpadded with XOR-swizzled 16-byte
@@ -340,7 +340,8 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 
     // ---- epilogue (all requests have landed and every wave is past its last fragment read)
     store_quadrant_bf16(acc, 1.0f, lds + w * kEpilogueScratchBytes,
-                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane);
+                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
+                        M - (m0 + wm * 128), N - (n0 + wn * 128));
 }
 
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
@@ -353,7 +354,10 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
     auto Bp = static_cast<const uint16_t*>(b);
     auto Cp = static_cast<uint16_t*>(c);
     // 32-bit buffer offsets: one 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
-    const bool fast_ok = !edge && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
+    // The fast kernel needs whole K slices; ragged M and N are handled by the zero fill of the
+    // buffer loads (rows past the end) and by the guarded epilogue (columns past N only ever
+    // contribute to outputs that are not stored).
+    const bool fast_ok = (K % BK == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N * 2 < ((size_t)1 << 32));
     if (fast_ok) {
 #define TYR_GEMM_FAST(TB)                                                                         \

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path for M % 256 == 0, N % 256 == 0, K % 128 == 0: slices go from global memory straight
+// Fast path for K % 128 == 0 (any M; N % 16 == 0): slices go from global memory straight
 // into LDS, unpadded rows with XOR-swizzled 16-byte chunks; a [K,N] B stays row-major in LDS and
 // its fragments (32 consecutive k for one n) are gathered with the byte-transposing LDS read.
 namespace gemm8f {
@@ -363,7 +363,8 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     }
 
     store_quadrant_bf16(acc, scale, lds + w * kEpilogueScratchBytes,
-                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane);
+                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
+                        M - (m0 + wm * 128), N - (n0 + wn * 128));
 }
 
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
@@ -376,7 +377,9 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
     auto Bp = static_cast<const uint8_t*>(bq);
     auto Cp = static_cast<uint16_t*>(c);
     // 32-bit buffer offsets: a 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
-    const bool fast_ok = !edge && (size_t)256 * K < ((size_t)1 << 31) &&
+    // The fast kernel needs whole K slices; ragged M and N are handled by the zero fill of the
+    // buffer loads and by the guarded epilogue.
+    const bool fast_ok = (K % BK == 0) && (size_t)256 * K < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N < ((size_t)1 << 32));
     if (fast_ok) {
 #define TYR_GEMM8_FAST(TB)                                                                        \
