@@ -5,11 +5,13 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The headline workload is the causal flash-attention forward the target is quoted on
-(bf16, B=16 H=16 N=4096 D=128); the other three configurations (GQA decode, bf16 GEMM, fp8 GEMM)
+(bf16, B=16 H=16 N=4096 D=128); the other configurations (attention backward, GQA decode, bf16 GEMM,
+fp8 GEMM)
 are measured in the same run and reported under "other_workloads" of the single JSON line.
 
 FLOP / byte conventions (algorithmic work, fixed per configuration):
   attn_fwd_causal : 4*B*H*N^2*D / 2 FLOP (two GEMMs, causal half)           -> MFMA bf16 2.5 PFLOP/s
+  attn_bwd_causal : 10*B*H*N^2*D / 2 FLOP (five GEMMs, causal half)         -> MFMA bf16 2.5 PFLOP/s
   gqa_decode      : bytes of K + V + Q + O                                   -> HBM 8 TB/s
   gemm_bf16       : 2*M*N*K FLOP                                             -> MFMA bf16 2.5 PFLOP/s
   gemm_fp8        : 2*M*N*K FLOP                                             -> MFMA fp8 5.0 PFLOP/s
@@ -94,6 +96,44 @@ def wl_attn(torch, tyr, steps, warmup, cpu):
                                "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"LibTorch CPU scaled_dot_product_attention(is_causal) on 1 of 16 batch "
                                          f"entries (16 heads, N=4096, D=128, bf16), {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_attn_bwd(torch, tyr, steps, warmup, cpu):
+    B, H, N, D = 16, 16, 4096, 128
+    torch.manual_seed(0)
+    q, k, v, g = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(4))
+    sc = 1.0 / math.sqrt(D)
+    o, lse = tyr.flash_attn_fwd(q, k, v, causal=True, scale=sc)
+    fn = lambda: tyr.flash_attn_bwd(q, k, v, o, lse, g, causal=True, scale=sc)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    flop = 10.0 * B * H * N * N * D / 2.0
+    tf = flop / (ms * 1e-3) / 1e12
+    res = {
+        "metric": "attn bwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+        "dtype": "bf16",
+        "config": {"workload": "causal flash-attention backward, bf16, B=16 H=16 N=4096 D=128, dQ + dK + dV",
+                   "flop_convention": "10*B*H*N^2*D/2 (five GEMMs, causal half); the two kernels execute seven",
+                   "scale": "1/sqrt(128)"},
+        "roofline": {"bound": "mfma", "kernel": "flash_attn_bwd_dq_kernel<128,true> + flash_attn_bwd_dkv_kernel<128,true>",
+                     "achieved": tf, "peak": PEAK["mfma_bf16"], "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"],
+                     "traffic": TRAFFIC.get("attn_bwd_causal")},
+    }
+    if cpu:
+        from oracle import libtorch_path as lt
+        hs = 4                                     # sample: 4 of the 256 heads
+        qc, kc, vc, gc = (t[:1, :hs].cpu() for t in (q, k, v, g))
+        lt.sdpa_4d_backward(qc[:, :1], kc[:, :1], vc[:, :1], gc[:, :1], True)   # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or (time.perf_counter() - t0 < 10 and reps < 20):
+            lt.sdpa_4d_backward(qc, kc, vc, gc, True)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": (14.0 * hs * N * N * D / 2.0) / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU autograd of scaled_dot_product_attention(is_causal), forward + "
+                                         f"backward (14*N^2*D/2 FLOP per head), f32, 4 heads of N=4096 D=128, "
+                                         f"{reps} reps, {dt * 1e3:.0f} ms each"}
     return res
 
 
@@ -221,7 +261,7 @@ def wl_copy(torch, tyr, steps, warmup, cpu):
                          "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": 2.0 * n}}
 
 
-WORKLOADS = {"attn_fwd_causal": wl_attn, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16, "gemm_fp8": wl_gemm_fp8}
+WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16, "gemm_fp8": wl_gemm_fp8}
 CALIBRATION = {"copy_1gib": wl_copy}
 
 

@@ -76,6 +76,33 @@ int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
                            int causal, float scale, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Flash-attention backward.
+ *
+ * Replaces the pair `tkMhaH100BwdPrep2Block` + `tkMhaH100Bwd2BlockPartials`
+ * (Tyr/GPU/Kernels/MhaH100.lean:197-344; launched from
+ * Examples/GPU/RunMhaH100.lean:118-140) for any B, H, N, and the host-side
+ * reduction of the per-(kv tile, q tile) partials that runner performs
+ * (Examples/GPU/RunMhaH100.lean:131-138): dK and dV come out final.  The
+ * values are the gradients autograd returns for
+ * `scaled_dot_product_attention` (Examples/GPU/RunMhaH100.lean:56-64).
+ *
+ *   q, k, v, o, d_o : bf16 [B, H, N, D] row-major contiguous; o and lse are the
+ *                     outputs of tyr_hip_flash_attn_fwd for the same q, k, v, causal, scale
+ *   lse             : f32 [B, H, N], natural log of the row sums of exp(scaled scores)
+ *   dq, dk, dv      : bf16 [B, H, N, D] (written; need not be initialised)
+ *   workspace       : device scratch of at least tyr_hip_flash_attn_bwd_workspace_bytes(...)
+ *                     bytes, 16-byte aligned; contents need not be initialised
+ * Supported: D in {64, 128}; any N >= 1 with N*D*2 < 2^31; B*H*ceil(N/128) < 2^31.
+ * The result is deterministic (no atomic accumulation).
+ */
+size_t tyr_hip_flash_attn_bwd_workspace_bytes(uint64_t B, uint64_t H, uint64_t N, uint64_t D);
+int tyr_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o,
+                           const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                           uint64_t B, uint64_t H, uint64_t N, uint64_t D,
+                           int causal, float scale, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* ---------------------------------------------------------------------------
  * GQA decode attention (one query token per sequence), split-KV + LSE combine.
  *
  * GPU twin of `lean_torch_sdpa_gqa_qkv` with q_seq = 1, is_causal = false,

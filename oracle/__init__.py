@@ -46,6 +46,8 @@ def lib() -> ctypes.CDLL:
                                  ctypes.c_void_p, ctypes.c_int)
         L.oracle_attn_fwd_f64.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
         L.oracle_attn_fwd_f64.restype = None
+        L.oracle_attn_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
+        L.oracle_attn_bwd_f64.restype = None
         L.oracle_attn_fwd_tiled.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f32, i64]
         L.oracle_attn_fwd_tiled.restype = None
         L.oracle_gqa_decode.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, f32, i64]
@@ -114,6 +116,16 @@ def attn_fwd_f64(q, k, v, causal: bool, scale: float):
     lse = np.empty((B, H, N), np.float32)
     lib().oracle_attn_fwd_f64(_p(q), _p(k), _p(v), _p(o), _p(lse), B, H, N, D, int(causal), float(scale))
     return o, lse
+
+
+def attn_bwd_f64(q, k, v, d_o, causal: bool, scale: float):
+    """Double-precision attention backward.  q,k,v,d_o uint16 [B,H,N,D] -> (dQ, dK, dV) f32."""
+    q, k, v, d_o = (_chk(t, np.uint16, n) for t, n in ((q, "q"), (k, "k"), (v, "v"), (d_o, "d_o")))
+    B, H, N, D = q.shape
+    dq, dk, dv = (np.empty((B, H, N, D), np.float32) for _ in range(3))
+    lib().oracle_attn_bwd_f64(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), B, H, N, D,
+                              int(causal), float(scale))
+    return dq, dk, dv
 
 
 def attn_fwd_tiled(q, k, v, causal: bool, scale: float, tile_kv: int = 64):

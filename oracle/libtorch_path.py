@@ -40,6 +40,17 @@ def sdpa_4d(q, k, v, is_causal: bool, dropout_p: float = 0.0):
     return F.scaled_dot_product_attention(q, k, v, None, dropout_p, is_causal)
 
 
+def sdpa_4d_backward(q, k, v, d_o, is_causal: bool):
+    """Gradients of sdpa_4d with respect to q, k, v for the upstream gradient d_o, taken from
+    autograd the way the reference's runner takes them (set_requires_grad, backward(out, dO),
+    grad_of).  Inputs are converted to f32 first so the result is the f32 gradient of the
+    rounded inputs."""
+    q32, k32, v32 = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    out = F.scaled_dot_product_attention(q32, k32, v32, None, 0.0, is_causal)
+    out.backward(d_o.float())
+    return q32.grad, k32.grad, v32.grad
+
+
 def sdpa_gqa_qkv(q, k, v, is_causal: bool = False, enable_gqa: bool = True, dropout_p: float = 0.0):
     n_head, n_kv_head = q.shape[1], k.shape[1]
     if enable_gqa and n_head != n_kv_head and n_kv_head > 0:

@@ -16,6 +16,12 @@
  *   oracle_attn_fwd_f64     textbook softmax(QK^T*scale + mask) V in double; the
  *                           same math as Examples/GPU/RunFlashAttn.lean:31-48
  *                           (reference values for O and LSE).
+ *   oracle_attn_bwd_f64     Tyr/GPU/Kernels/MhaH100.lean:197-344 (backward prep
+ *                           d = rowsum(dO o O) and the dQ / dK / dV products:
+ *                           P = exp(S*scale - lse), dP = dO V^T, dS = P o (dP - d),
+ *                           dV = P^T dO, dK = scale dS^T Q, dQ = scale dS K), in
+ *                           double; reference values as Examples/GPU/RunMhaH100.lean:56-64
+ *                           takes them from autograd.
  *   oracle_gqa_decode       cc/src/tyr.cpp:4100-4133 (repeat_interleave mapping),
  *                           Tyr/GPU/Kernels/FlashAttn3.lean:535-624 (q-head packing),
  *                           split/merge algebra of Tyr/GPU/Kernels/RingAttn.lean
@@ -137,6 +143,65 @@ void oracle_attn_fwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v
             if (lse) lse[bh * N + i] = (float)(log(l) + m);
             free(s);
         }
+    }
+}
+
+/* Attention backward in double precision.  q,k,v,d_o: bf16 bit patterns [B,H,N,D];
+ * dq,dk,dv: f32 [B,H,N,D].  The forward quantities (P, O) are recomputed here in double,
+ * so the result is the exact gradient of oracle_attn_fwd_f64's O contracted with d_o. */
+void oracle_attn_bwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                         const uint16_t* d_o, float* dq, float* dk, float* dv,
+                         int64_t B, int64_t H, int64_t N, int64_t D,
+                         int causal, double scale) {
+    #pragma omp parallel for schedule(dynamic)
+    for (int64_t bh = 0; bh < B * H; ++bh) {
+        const uint16_t* qh = q + bh * N * D;
+        const uint16_t* kh = k + bh * N * D;
+        const uint16_t* vh = v + bh * N * D;
+        const uint16_t* gh = d_o + bh * N * D;
+        double* dka = (double*)calloc((size_t)(N * D), sizeof(double));
+        double* dva = (double*)calloc((size_t)(N * D), sizeof(double));
+        double* p = (double*)malloc(sizeof(double) * (size_t)N);
+        double* dp = (double*)malloc(sizeof(double) * (size_t)N);
+        double* dqa = (double*)malloc(sizeof(double) * (size_t)D);
+        for (int64_t i = 0; i < N; ++i) {
+            const int64_t jmax = causal ? i + 1 : N;
+            double m = -INFINITY;
+            for (int64_t j = 0; j < jmax; ++j) {
+                double acc = 0.0;
+                for (int64_t d = 0; d < D; ++d)
+                    acc += (double)bf16_to_f32(qh[i * D + d]) * (double)bf16_to_f32(kh[j * D + d]);
+                p[j] = acc * scale;
+                if (p[j] > m) m = p[j];
+            }
+            double l = 0.0;
+            for (int64_t j = 0; j < jmax; ++j) { p[j] = exp(p[j] - m); l += p[j]; }
+            for (int64_t j = 0; j < jmax; ++j) p[j] /= l;
+            /* dP_j = dO_i . V_j ; delta = sum_j P_j dP_j  (= dO_i . O_i) */
+            double delta = 0.0;
+            for (int64_t j = 0; j < jmax; ++j) {
+                double acc = 0.0;
+                for (int64_t d = 0; d < D; ++d)
+                    acc += (double)bf16_to_f32(gh[i * D + d]) * (double)bf16_to_f32(vh[j * D + d]);
+                dp[j] = acc;
+                delta += p[j] * acc;
+            }
+            for (int64_t d = 0; d < D; ++d) dqa[d] = 0.0;
+            for (int64_t j = 0; j < jmax; ++j) {
+                const double ds = p[j] * (dp[j] - delta) * scale;
+                for (int64_t d = 0; d < D; ++d) {
+                    dqa[d] += ds * (double)bf16_to_f32(kh[j * D + d]);
+                    dka[j * D + d] += ds * (double)bf16_to_f32(qh[i * D + d]);
+                    dva[j * D + d] += p[j] * (double)bf16_to_f32(gh[i * D + d]);
+                }
+            }
+            for (int64_t d = 0; d < D; ++d) dq[(bh * N + i) * D + d] = (float)dqa[d];
+        }
+        for (int64_t x = 0; x < N * D; ++x) {
+            dk[bh * N * D + x] = (float)dka[x];
+            dv[bh * N * D + x] = (float)dva[x];
+        }
+        free(dka); free(dva); free(p); free(dp); free(dqa);
     }
 }
 

@@ -1,0 +1,540 @@
+// Flash-attention backward for gfx950 (bf16 in, f32 accumulation, bf16 dQ / dK / dV).
+//
+// Arithmetic contract of the reference (Tyr/GPU/Kernels/MhaH100.lean):
+//   :197-232  backward prep      delta[i] = sum_d dO[i,d] * O[i,d]
+//   :234-344  backward           S = Q K^T * scale ; P = exp(S - lse) ; dP = dO V^T ;
+//                                dS = P o (dP - delta) ; dV += bf16(P)^T dO ;
+//                                dK += bf16(dS)^T Q * scale ; dQ += bf16(dS) K * scale
+// (expected values in the reference's runner come from autograd of scaled_dot_product_attention,
+// Examples/GPU/RunMhaH100.lean:56-64).  exp is evaluated as exp2 with log2(e) folded into the
+// scale and into the saved log-sum-exp.  causal: key j visible to query i iff j <= i.
+//
+// Two kernels, no atomics, every output written once (results are deterministic):
+//
+//  1. flash_attn_bwd_dq_kernel: one workgroup = 128 query rows (4 waves x 32 rows), keys/values
+//     stream through LDS in tiles of 64 rows exactly as in the forward kernel.  Products are
+//     computed transposed so that every lane owns one query column:
+//        S^T  (64 kv x 32 q) = K_tile x Q^T       dP^T (64 kv x 32 q) = V_tile x dO^T
+//        dQ^T (D x 32 q)    += K_tile^T x dS^T
+//     so lse and delta are per-lane scalars and dS^T is already in the register slots the third
+//     product wants as its column operand.  The prologue also computes delta (each wave holds its
+//     dO rows and reads its O rows once) and writes (lse * log2 e, delta) pairs to the workspace
+//     for the second kernel; rows of the padding up to a multiple of 128 get (+inf, 0), which
+//     makes their probabilities exactly zero.
+//
+//  2. flash_attn_bwd_dkv_kernel: one workgroup = 128 key rows (4 waves x 32 rows, K and V
+//     fragments of those rows live in registers), queries / dO stream through LDS in tiles of 64
+//     rows, three stages deep.  Every lane owns one key column:
+//        S  (32 q x 32 kv) = Q_tile x K_w^T        dP (32 q x 32 kv) = dO_tile x V_w^T
+//        dV^T (D x 32 kv) += dO_tile^T x P         dK^T (D x 32 kv) += Q_tile^T x dS
+//     with lse / delta of the 16 query rows a lane holds read from the staged pairs.
+//
+// Both recompute S (7 matrix products for an algorithm that needs 5): the price of writing dQ
+// without a float atomic accumulation buffer and a conversion pass.
+//
+// LDS tiles are row-major with 16-byte chunks XOR-swizzled by a function of the row that is
+// conflict-free both for row fragments (16-byte reads, lane = row) and for transposed fragments
+// (ds_read_b64_tr_b16 over 4 rows x 64 bytes per lane-group pair).
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace tyr {
+
+namespace fab {
+constexpr int THREADS = 256;
+constexpr float LOG2E = 1.4426950408889634f;
+
+// chunk index within a row -> stored chunk index.  The mask is a bijection of (row mod 16) [of
+// ((row / 2) mod 8) for 128-byte rows], so 16 consecutive rows put one logical chunk on 16
+// different bank groups; its upper bits follow row mod 4, which spreads the 4 rows a lane group
+// of the transposing read touches over the 4 64-byte quarters of the bank space.
+template <int D> __device__ __forceinline__ int swz(int row, int c) {
+    return D == 128 ? (c ^ (((row & 3) << 2) | ((row >> 2) & 3)))
+                    : (c ^ ((((row >> 1) & 1) << 2) | ((row >> 2) & 3)));
+}
+
+template <int D>
+struct CfgQ {                                       // dQ kernel
+    static constexpr int BM = 128, BN = 64;
+    static constexpr int ROW = D * 2, KCH = D / 8;
+    static constexpr int TILE = BN * ROW;
+    static constexpr int V_BASE = 2 * TILE;         // K stage 0, K stage 1, V stage 0, V stage 1
+    static constexpr int LDS = 4 * TILE;
+    static constexpr int PT = BN * KCH / THREADS;   // 16-byte chunks per thread per tile
+    static constexpr int KSTEPS = D / 16, DT = D / 32;
+};
+
+template <int D>
+struct CfgK {                                       // dK / dV kernel
+    static constexpr int BNK = 128, BQ = 64, NST = 3;
+    static constexpr int ROW = D * 2, KCH = D / 8;
+    static constexpr int TILE = BQ * ROW;
+    static constexpr int STAT = 1024;               // 64 (lse2, delta) pairs + slack of one load
+    static constexpr int STAGE = 2 * TILE + STAT;   // Q tile, dO tile, pairs
+    static constexpr int LDS = NST * STAGE;
+    static constexpr int PT = BQ * KCH / THREADS;
+    static constexpr int KSTEPS = D / 16, DT = D / 32;
+    static constexpr int LOADS_PER_TILE = 2 * PT + 1;
+};
+
+__device__ __forceinline__ float dot8_bf16(u32x4 a, u32x4 b) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s += bf16_lo(a[i]) * bf16_lo(b[i]) + bf16_hi(a[i]) * bf16_hi(b[i]);
+    return s;
+}
+
+// One wave's 32 columns x D rows accumulator (lane = column l%32, register e of tile dt <-> row
+// 32 dt + 8(e/4) + 4(l/32) + e%4), scaled, written as bf16 rows of length D: out row = column.
+// Goes through a private LDS scratch so the global stores are 16 bytes per lane along rows.
+template <int D>
+__device__ __forceinline__ void store_transposed_bf16(const f32x16 (&acc)[D / 32], float mul, unsigned char* scratch,
+                                                      uint16_t* out_rows, int rows_valid, int lane) {
+    constexpr int SROW = D * 2 + 16;
+    const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x2 v;
+            v.x = pack_bf16(acc[dt][4 * q4 + 0] * mul, acc[dt][4 * q4 + 1] * mul);
+            v.y = pack_bf16(acc[dt][4 * q4 + 2] * mul, acc[dt][4 * q4 + 3] * mul);
+            *reinterpret_cast<u32x2*>(scratch + r * SROW + (dt * 32 + q4 * 8 + g * 4) * 2) = v;
+        }
+    }
+    constexpr int CH = D / 8;
+    constexpr int RPI = 64 / CH;
+#pragma unroll
+    for (int k = 0; k < 32 / RPI; ++k) {
+        const int row = lane / CH + RPI * k;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * SROW + (lane % CH) * 16);
+        if (row < rows_valid) st_global_16(out_rows + (size_t)row * D + (lane % CH) * 8, v);
+    }
+}
+}  // namespace fab
+
+// ------------------------------------------------------------------------------------------
+// dQ (and the (lse2, delta) pairs)
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
+    const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
+    const uint16_t* __restrict__ O, const uint16_t* __restrict__ dO, const float* __restrict__ LSE,
+    uint16_t* __restrict__ dQ, float2* __restrict__ stats, int BH, int N, int ntq, float scale,
+    float scale_log2) {
+    using namespace fab;
+    using C = CfgQ<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r = lane & 31, g = lane >> 5;
+
+    int bh, qt;
+    {
+        const int id = blockIdx.x;
+        int tr;
+        if ((BH & 7) == 0) {
+            const int xcd = id & 7, slot = id >> 3;
+            bh = (slot / ntq) * 8 + xcd;
+            tr = slot % ntq;
+        } else {
+            bh = id / ntq;
+            tr = id % ntq;
+        }
+        qt = CAUSAL ? ntq - 1 - tr : tr;
+    }
+    const int q0 = qt * C::BM;
+    const int qw0 = q0 + w * 32;
+    const size_t head_off = (size_t)bh * N * D;
+    const uint16_t* Kh = Kp + head_off;
+    const uint16_t* Vh = Vp + head_off;
+    const int kv_end = CAUSAL ? min(N, q0 + C::BM) : N;
+    const int nkv = (kv_end + C::BN - 1) / C::BN;
+    const int qpos = qw0 + r;
+
+    // ---- this wave's Q^T and dO^T fragments (lane = query row, columns 16i + 8g + [0,8)),
+    //      delta = dO . O and lse in log2 units
+    bf16x8 qf[C::KSTEPS], dof[C::KSTEPS];
+    float delta, lse2;
+    {
+        const int qrow = min(qpos, N - 1);
+        const size_t off = head_off + (size_t)qrow * D + g * 8;
+        float part = 0.0f;
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) {
+            qf[i] = __builtin_bit_cast(bf16x8, ld_global_16(Q + off + i * 16));
+            const u32x4 dv = ld_global_16(dO + off + i * 16);
+            const u32x4 ov = ld_global_16(O + off + i * 16);
+            dof[i] = __builtin_bit_cast(bf16x8, dv);
+            part += dot8_bf16(dv, ov);
+        }
+        delta = part + xor32(part);
+        lse2 = LSE[(size_t)bh * N + qrow] * LOG2E;
+        if (g == 0) {
+            const size_t npad = (size_t)ntq * C::BM;
+            stats[(size_t)bh * npad + qpos] = qpos < N ? make_float2(lse2, delta) : make_float2(INFINITY, 0.0f);
+        }
+    }
+
+    // ---- K / V tile loaders (global memory straight into LDS, swizzle applied on the global side)
+    const uint32_t head_bytes = (uint32_t)N * D * 2u;
+    const u32x4 k_rsrc = make_raw_rsrc(Kh, head_bytes);
+    const u32x4 v_rsrc = make_raw_rsrc(Vh, head_bytes);
+    constexpr int ROWS_PER_INST = 1024 / C::ROW;
+    int g_voff[C::PT];
+#pragma unroll
+    for (int m = 0; m < C::PT; ++m) {
+        const int row = (w * C::PT + m) * ROWS_PER_INST + lane / C::KCH;
+        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16;
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PT * 1024u);
+    auto issue_kv = [&](int stage, int j0) {
+        const uint32_t dst = wave_dst + (uint32_t)stage * C::TILE;
+#pragma unroll
+        for (int m = 0; m < C::PT; ++m) {
+            load_global_to_lds_16(k_rsrc, dst + m * 1024, g_voff[m], j0 * C::ROW);
+            load_global_to_lds_16(v_rsrc, dst + C::V_BASE + m * 1024, g_voff[m], j0 * C::ROW);
+        }
+    };
+
+    // row fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g
+    int row_off[C::KSTEPS];
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) row_off[i] = r * C::ROW + swz<D>(r, 2 * i + g) * 16;
+    // transposed fragment (d tile dt; kv rows 16c + 8h + 4g + [0,4)): as a source lane of the
+    // transposing read this lane points at row 4(b/2) + (lane%16)/4 (+8 for the second read),
+    // 8 bytes at d = 32dt + 16(b&1) + 4(lane%4), b = lane/16.
+    int tr_lo[C::DT], tr_hi[C::DT];
+    {
+        const int i16 = lane & 15, b16 = lane >> 4;
+        const int row = 4 * (b16 >> 1) + (i16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+            const int dcol = 32 * dt + 16 * (b16 & 1) + 4 * (i16 & 3);
+            tr_lo[dt] = row * C::ROW + swz<D>(row, dcol >> 3) * 16 + (dcol & 7) * 2;
+            tr_hi[dt] = (row + 8) * C::ROW + swz<D>(row + 8, dcol >> 3) * 16 + (dcol & 7) * 2;
+        }
+    }
+
+    f32x16 dq[C::DT];
+#pragma unroll
+    for (int i = 0; i < C::DT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dq[i][e] = 0.0f;
+
+    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / C::BN + 1) : nkv;
+
+    issue_kv(0, 0);
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(qf[i]); pin_registers(dof[i]); }
+    wait_vmcnt0();
+    __syncthreads();
+
+    for (int j = 0; j < nkv; ++j) {
+        const int j0 = j * C::BN;
+        if (j + 1 < nkv) issue_kv((j + 1) & 1, j0 + C::BN);
+        if (j < nkv_w) {
+            const unsigned char* Kt = lds + (j & 1) * C::TILE;
+            const unsigned char* Vt = Kt + C::V_BASE;
+            f32x16 s[2], dp[2];
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
+#pragma unroll
+            for (int i = 0; i < C::KSTEPS; ++i) {
+#pragma unroll
+                for (int T = 0; T < 2; ++T) {
+                    const bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
+                    s[T] = mfma_32x32x16_bf16(ka, qf[i], s[T]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < C::KSTEPS; ++i) {
+#pragma unroll
+                for (int T = 0; T < 2; ++T) {
+                    const bf16x8 va = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
+                    dp[T] = mfma_32x32x16_bf16(va, dof[i], dp[T]);
+                }
+            }
+            // mask (diagonal tiles, ragged tail): register e of sub-tile T is kv row
+            // j0 + 32T + 8(e/4) + 4g + e%4
+            const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > N);
+            if (need_mask) {
+                const int lim = CAUSAL ? min(qpos, N - 1) : N - 1;
+                const int base = j0 + 4 * g;
+#pragma unroll
+                for (int T = 0; T < 2; ++T)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
+                        if (kv > lim) s[T][e] = -INFINITY;
+                    }
+            }
+            // dS^T = P^T o (dP^T - delta), packed into column-operand slots (group c = 2T + sh
+            // holds registers 8sh .. 8sh+7 of sub-tile T)
+            bf16x8 dsf[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int T = c >> 1, sh = c & 1;
+                u32x4 pk;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int e = 8 * sh + 2 * jj;
+                    const float p0 = fast_exp2(fmaf(s[T][e], scale_log2, -lse2));
+                    const float p1 = fast_exp2(fmaf(s[T][e + 1], scale_log2, -lse2));
+                    pk[jj] = pack_bf16(p0 * (dp[T][e] - delta), p1 * (dp[T][e + 1] - delta));
+                }
+                dsf[c] = __builtin_bit_cast(bf16x8, pk);
+            }
+            // dQ^T += K^T dS^T
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt) {
+                    const bf16x4 lo = ds_read_tr16(Kt + tr_lo[dt] + c * 16 * C::ROW);
+                    const bf16x4 hi = ds_read_tr16(Kt + tr_hi[dt] + c * 16 * C::ROW);
+                    const bf16x8 kt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
+                }
+            }
+        }
+        wait_vmcnt0();
+        __syncthreads();
+    }
+
+    store_transposed_bf16<D>(dq, scale, lds + w * (32 * (D * 2 + 16)), dQ + head_off + (size_t)qw0 * D,
+                             N - qw0, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// dK, dV
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
+    const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
+    const uint16_t* __restrict__ dO, const float2* __restrict__ stats, uint16_t* __restrict__ dK,
+    uint16_t* __restrict__ dV, int BH, int N, int ntk, int npad, float scale, float scale_log2) {
+    using namespace fab;
+    using C = CfgK<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r = lane & 31, g = lane >> 5;
+
+    int bh, kt;
+    {
+        const int id = blockIdx.x;
+        if ((BH & 7) == 0) {
+            const int xcd = id & 7, slot = id >> 3;
+            bh = (slot / ntk) * 8 + xcd;
+            kt = slot % ntk;              // causal: key tile 0 meets every query tile, so heavy first
+        } else {
+            bh = id / ntk;
+            kt = id % ntk;
+        }
+    }
+    const int n0 = kt * C::BNK;
+    const int nw0 = n0 + w * 32;
+    const int kvpos = nw0 + r;
+    const size_t head_off = (size_t)bh * N * D;
+
+    // ---- this wave's K and V rows as column operands (lane = key row, columns 16i + 8g + [0,8))
+    bf16x8 kf[C::KSTEPS], vf[C::KSTEPS];
+    {
+        const size_t off = head_off + (size_t)min(kvpos, N - 1) * D + g * 8;
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) {
+            kf[i] = __builtin_bit_cast(bf16x8, ld_global_16(Kp + off + i * 16));
+            vf[i] = __builtin_bit_cast(bf16x8, ld_global_16(Vp + off + i * 16));
+        }
+    }
+
+    // ---- Q / dO / pair tile loaders
+    const uint32_t head_bytes = (uint32_t)N * D * 2u;
+    const u32x4 q_rsrc = make_raw_rsrc(Q + head_off, head_bytes);
+    const u32x4 do_rsrc = make_raw_rsrc(dO + head_off, head_bytes);
+    const uint32_t stat_bytes = (uint32_t)npad * 8u;
+    const u32x4 st_rsrc = make_raw_rsrc(stats + (size_t)bh * npad, stat_bytes);
+    constexpr int ROWS_PER_INST = 1024 / C::ROW;
+    int g_voff[C::PT];
+#pragma unroll
+    for (int m = 0; m < C::PT; ++m) {
+        const int row = (w * C::PT + m) * ROWS_PER_INST + lane / C::KCH;
+        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16;
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PT * 1024u);
+    const int nq = (N + C::BQ - 1) / C::BQ;
+    // Tiles past the end are requested at an offset beyond the buffer (they read as zero), so that
+    // every iteration issues the same number of loads and the wait count below stays constant.
+    auto issue_tile = [&](int stage, int jq) {
+        const uint32_t dst = wave_dst + (uint32_t)stage * C::STAGE;
+        const bool live = jq < nq;
+        const int soff = live ? jq * C::BQ * C::ROW : (int)head_bytes;
+        const int ssoff = live ? jq * C::BQ * 8 : (int)stat_bytes;
+#pragma unroll
+        for (int m = 0; m < C::PT; ++m) {
+            load_global_to_lds_16(q_rsrc, dst + m * 1024, g_voff[m], soff);
+            load_global_to_lds_16(do_rsrc, dst + C::TILE + m * 1024, g_voff[m], soff);
+        }
+        // every wave requests the same kilobyte of pairs (identical bytes, one instruction)
+        load_global_to_lds_16(st_rsrc, lds_base + (uint32_t)stage * C::STAGE + 2 * C::TILE, lane * 16, ssoff);
+    };
+
+    int row_off[C::KSTEPS];
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) row_off[i] = r * C::ROW + swz<D>(r, 2 * i + g) * 16;
+    int tr_lo[C::DT], tr_hi[C::DT];
+    {
+        const int i16 = lane & 15, b16 = lane >> 4;
+        const int row = 4 * (b16 >> 1) + (i16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+            const int dcol = 32 * dt + 16 * (b16 & 1) + 4 * (i16 & 3);
+            tr_lo[dt] = row * C::ROW + swz<D>(row, dcol >> 3) * 16 + (dcol & 7) * 2;
+            tr_hi[dt] = (row + 8) * C::ROW + swz<D>(row + 8, dcol >> 3) * 16 + (dcol & 7) * 2;
+        }
+    }
+
+    f32x16 dk[C::DT], dv[C::DT];
+#pragma unroll
+    for (int i = 0; i < C::DT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { dk[i][e] = 0.0f; dv[i][e] = 0.0f; }
+
+    const int jq0 = CAUSAL ? n0 / C::BQ : 0;
+    const int ntile = nq - jq0;
+
+#pragma unroll
+    for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(kf[i]); pin_registers(vf[i]); }
+    issue_tile(0, jq0);
+    issue_tile(1, jq0 + 1);
+
+    int st = 0;
+    for (int it = 0; it < ntile; ++it) {
+        // all but the most recent tile's requests have landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::LOADS_PER_TILE) : "memory");
+        __syncthreads();
+        {
+            const int st2 = st + 2 >= C::NST ? st + 2 - C::NST : st + 2;
+            issue_tile(st2, jq0 + it + 2);
+        }
+        const int q0 = (jq0 + it) * C::BQ;
+        const unsigned char* Qt = lds + st * C::STAGE;
+        const unsigned char* dOt = Qt + C::TILE;
+        const unsigned char* St = Qt + 2 * C::TILE;
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const int qs0 = q0 + 32 * T;
+            if (CAUSAL && qs0 + 31 < nw0) continue;          // every query of the sub-tile precedes every key of the wave
+            f32x16 s, dp;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) { s[e] = 0.0f; dp[e] = 0.0f; }
+#pragma unroll
+            for (int i = 0; i < C::KSTEPS; ++i) {
+                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qt + row_off[i] + T * 32 * C::ROW);
+                s = mfma_32x32x16_bf16(qa, kf[i], s);
+                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOt + row_off[i] + T * 32 * C::ROW);
+                dp = mfma_32x32x16_bf16(da, vf[i], dp);
+            }
+            // register e <-> query row qs0 + 8(e/4) + 4g + e%4 ; its (lse2, delta) pair sits at
+            // pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte
+            const bool need_mask = CAUSAL && (qs0 < nw0 + 31);
+            bf16x8 pf[2], dsf[2];
+#pragma unroll
+            for (int sh = 0; sh < 2; ++sh) {
+                u32x4 ppk, dpk;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {                // e/4 = 2sh + h
+                    const int prow = 32 * T + 8 * (2 * sh + h) + 4 * g;
+                    const f32x4 a = *reinterpret_cast<const f32x4*>(St + prow * 8);
+                    const f32x4 b = *reinterpret_cast<const f32x4*>(St + prow * 8 + 16);
+                    const float l2[4] = {a[0], a[2], b[0], b[2]};
+                    const float dl[4] = {a[1], a[3], b[1], b[3]};
+                    float p[4], ds[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int e = 8 * sh + 4 * h + x;
+                        float pv = fast_exp2(fmaf(s[e], scale_log2, -l2[x]));
+                        if (need_mask && kvpos > qs0 + 8 * (2 * sh + h) + 4 * g + x) pv = 0.0f;
+                        p[x] = pv;
+                        ds[x] = pv * (dp[e] - dl[x]);
+                    }
+                    ppk[2 * h] = pack_bf16(p[0], p[1]);
+                    ppk[2 * h + 1] = pack_bf16(p[2], p[3]);
+                    dpk[2 * h] = pack_bf16(ds[0], ds[1]);
+                    dpk[2 * h + 1] = pack_bf16(ds[2], ds[3]);
+                }
+                pf[sh] = __builtin_bit_cast(bf16x8, ppk);
+                dsf[sh] = __builtin_bit_cast(bf16x8, dpk);
+            }
+            // dV^T += dO^T P ; dK^T += Q^T dS   (k-step c = 2T + sh: query rows 16c + 8h + 4g + [0,4))
+#pragma unroll
+            for (int sh = 0; sh < 2; ++sh) {
+                const int c = 2 * T + sh;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt) {
+                    const bf16x4 lo = ds_read_tr16(dOt + tr_lo[dt] + c * 16 * C::ROW);
+                    const bf16x4 hi = ds_read_tr16(dOt + tr_hi[dt] + c * 16 * C::ROW);
+                    dv[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf[sh], dv[dt]);
+                    const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
+                    const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
+                    dk[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7), dsf[sh], dk[dt]);
+                }
+            }
+        }
+        st = st + 1 == C::NST ? 0 : st + 1;
+    }
+    wait_vmcnt0();
+    __syncthreads();
+
+    unsigned char* scratch = lds + w * (32 * (D * 2 + 16));
+    store_transposed_bf16<D>(dv, 1.0f, scratch, dV + head_off + (size_t)nw0 * D, N - nw0, lane);
+    store_transposed_bf16<D>(dk, scale, scratch, dK + head_off + (size_t)nw0 * D, N - nw0, lane);
+}
+
+size_t flash_attn_bwd_workspace_bytes(int B, int H, int N) {
+    const size_t npad = (size_t)((N + 127) / 128) * 128;
+    return (size_t)B * H * npad * sizeof(float2);
+}
+
+int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                          const float* lse, void* dq, void* dk, void* dv, int B, int H, int N, int D,
+                          int causal, float scale, void* workspace, hipStream_t stream) {
+    using namespace fab;
+    const int BH = B * H;
+    const int ntq = (N + 127) / 128;
+    const int npad = ntq * 128;
+    dim3 grid((unsigned)(BH * ntq)), block(THREADS);
+    const float scale_log2 = scale * LOG2E;
+    auto Qp = static_cast<const uint16_t*>(q);
+    auto Kp = static_cast<const uint16_t*>(k);
+    auto Vp = static_cast<const uint16_t*>(v);
+    auto Op = static_cast<const uint16_t*>(o);
+    auto dOp = static_cast<const uint16_t*>(d_o);
+    auto st = static_cast<float2*>(workspace);
+#define TYR_FAB_LAUNCH(DD, CC)                                                                        \
+    do {                                                                                              \
+        static const hipError_t a1 = hipFuncSetAttribute(                                             \
+            reinterpret_cast<const void*>(&flash_attn_bwd_dq_kernel<DD, CC>),                         \
+            hipFuncAttributeMaxDynamicSharedMemorySize, CfgQ<DD>::LDS);                               \
+        static const hipError_t a2 = hipFuncSetAttribute(                                             \
+            reinterpret_cast<const void*>(&flash_attn_bwd_dkv_kernel<DD, CC>),                        \
+            hipFuncAttributeMaxDynamicSharedMemorySize, CfgK<DD>::LDS);                               \
+        if (a1 != hipSuccess || a2 != hipSuccess) return -1;                                          \
+        hipLaunchKernelGGL((flash_attn_bwd_dq_kernel<DD, CC>), grid, block, CfgQ<DD>::LDS, stream,    \
+                           Qp, Kp, Vp, Op, dOp, lse, static_cast<uint16_t*>(dq), st, BH, N, ntq,      \
+                           scale, scale_log2);                                                        \
+        hipLaunchKernelGGL((flash_attn_bwd_dkv_kernel<DD, CC>), grid, block, CfgK<DD>::LDS, stream,   \
+                           Qp, Kp, Vp, dOp, st, static_cast<uint16_t*>(dk),                           \
+                           static_cast<uint16_t*>(dv), BH, N, ntq, npad, scale, scale_log2);          \
+    } while (0)
+    if (D == 128) { if (causal) TYR_FAB_LAUNCH(128, true); else TYR_FAB_LAUNCH(128, false); }
+    else          { if (causal) TYR_FAB_LAUNCH(64, true);  else TYR_FAB_LAUNCH(64, false); }
+#undef TYR_FAB_LAUNCH
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace tyr

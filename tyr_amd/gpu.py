@@ -85,6 +85,33 @@ def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, str
     return o, lse
 
 
+def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | None = None, stream=None):
+    """dQ, dK, dV = flashAttnBwd q k v o lse dO causal scale.
+
+    q, k, v, o, d_o bf16 [B,H,N,D]; lse f32 [B,H,N]; o and lse as returned by flash_attn_fwd for
+    the same q, k, v, causal and scale.  Returns three bf16 [B,H,N,D] tensors."""
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "dO")):
+        _check(t, n, torch.bfloat16, 4)
+        if t.shape != q.shape:
+            raise TyrGpuError("q, k, v, o, dO must have the same shape [B, H, N, D]")
+    _check(lse, "lse", torch.float32, 3)
+    B, H, N, D = q.shape
+    if tuple(lse.shape) != (B, H, N):
+        raise TyrGpuError("lse must have shape [B, H, N]")
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    nbytes = lib.tyr_hip_flash_attn_bwd_workspace_bytes(B, H, N, D)
+    ws = torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=q.device)
+    rc = lib.tyr_hip_flash_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
+                                    lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D,
+                                    int(bool(causal)), float(scale), ws.data_ptr(), ws.numel(),
+                                    _stream(stream))
+    _raise(rc, "flashAttnBwd")
+    return dq, dk, dv
+
+
 def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len: int | None = None,
                stream=None):
     """O, LSE = gqaDecode q k v scale numSplits.
