@@ -24,7 +24,7 @@
 //
 //  2. flash_attn_bwd_dkv_kernel: one workgroup = 128 key rows (4 waves x 32 rows, K and V
 //     fragments of those rows live in registers), queries / dO stream through LDS in tiles of 64
-//     rows, three stages deep.  Every lane owns one key column:
+//     rows, four stages deep.  Every lane owns one key column:
 //        S  (32 q x 32 kv) = Q_tile x K_w^T        dP (32 q x 32 kv) = dO_tile x V_w^T
 //        dV^T (D x 32 kv) += dO_tile^T x P         dK^T (D x 32 kv) += Q_tile^T x dS
 //     with lse / delta of the 16 query rows a lane holds read from the staged pairs.
@@ -35,6 +35,8 @@
 // LDS tiles are row-major with 16-byte chunks XOR-swizzled by a function of the row that is
 // conflict-free both for row fragments (16-byte reads, lane = row) and for transposed fragments
 // (ds_read_b64_tr_b16 over 4 rows x 64 bytes per lane-group pair).
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -66,7 +68,7 @@ struct CfgQ {                                       // dQ kernel
 
 template <int D>
 struct CfgK {                                       // dK / dV kernel
-    static constexpr int BNK = 128, BQ = 64, NST = 3;
+    static constexpr int BNK = 128, BQ = 64, NST = 4;   // NST must stay a power of two
     static constexpr int ROW = D * 2, KCH = D / 8;
     static constexpr int TILE = BQ * ROW;
     static constexpr int STAT = 1024;               // 64 (lse2, delta) pairs + slack of one load
@@ -407,85 +409,121 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const int jq0 = CAUSAL ? n0 / C::BQ : 0;
     const int ntile = nq - jq0;
 
+    // S and dP of one 32-row sub-tile T of the tile staged at Qt / dOt
+    auto scores = [&](const unsigned char* Qt, const unsigned char* dOt, int T, f32x16& s, f32x16& dp) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { s[e] = 0.0f; dp[e] = 0.0f; }
+        bf16x8 qa[C::KSTEPS], da[C::KSTEPS];          // all row fragments are requested up front
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) {
+            qa[i] = *reinterpret_cast<const bf16x8*>(Qt + row_off[i] + T * 32 * C::ROW);
+            da[i] = *reinterpret_cast<const bf16x8*>(dOt + row_off[i] + T * 32 * C::ROW);
+        }
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) {
+            s = mfma_32x32x16_bf16(qa[i], kf[i], s);
+            dp = mfma_32x32x16_bf16(da[i], vf[i], dp);
+        }
+    };
+    // P and dS of that sub-tile as column operands.  Register e <-> query row qs0 + 8(e/4) + 4g +
+    // e%4; its (lse2, delta) pair sits at pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte.
+    auto probabilities = [&](auto masked, const unsigned char* St, int T, int qs0, const f32x16& s,
+                             const f32x16& dp, bf16x8 (&pf)[2], bf16x8 (&dsf)[2]) {
+        constexpr bool need_mask = decltype(masked)::value;
+#pragma unroll
+        for (int sh = 0; sh < 2; ++sh) {
+            u32x4 ppk, dpk;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {                // e/4 = 2sh + h
+                const int prow = 32 * T + 8 * (2 * sh + h) + 4 * g;
+                const f32x4 a = *reinterpret_cast<const f32x4*>(St + prow * 8);
+                const f32x4 b = *reinterpret_cast<const f32x4*>(St + prow * 8 + 16);
+                const float l2[4] = {a[0], a[2], b[0], b[2]};
+                const float dl[4] = {a[1], a[3], b[1], b[3]};
+                float p[4], ds[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
+                if (need_mask) {                         // only tiles that touch the diagonal
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (kvpos > qs0 + 8 * (2 * sh + h) + 4 * g + x) p[x] = 0.0f;
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) ds[x] = p[x] * (dp[8 * sh + 4 * h + x] - dl[x]);
+                ppk[2 * h] = pack_bf16(p[0], p[1]);
+                ppk[2 * h + 1] = pack_bf16(p[2], p[3]);
+                dpk[2 * h] = pack_bf16(ds[0], ds[1]);
+                dpk[2 * h + 1] = pack_bf16(ds[2], ds[3]);
+            }
+            pf[sh] = __builtin_bit_cast(bf16x8, ppk);
+            dsf[sh] = __builtin_bit_cast(bf16x8, dpk);
+        }
+    };
+    // dV^T += dO^T P ; dK^T += Q^T dS   (k-step c = 2T + sh: query rows 16c + 8h + 4g + [0,4))
+    auto accumulate = [&](const unsigned char* Qt, const unsigned char* dOt, int T, const bf16x8 (&pf)[2],
+                          const bf16x8 (&dsf)[2]) {
+#pragma unroll
+        for (int sh = 0; sh < 2; ++sh) {
+            const int c = 2 * T + sh;
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt) {
+                const bf16x4 lo = ds_read_tr16(dOt + tr_lo[dt] + c * 16 * C::ROW);
+                const bf16x4 hi = ds_read_tr16(dOt + tr_hi[dt] + c * 16 * C::ROW);
+                dv[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf[sh], dv[dt]);
+                const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
+                const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
+                dk[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7), dsf[sh], dk[dt]);
+            }
+        }
+    };
+
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(kf[i]); pin_registers(vf[i]); }
     issue_tile(0, jq0);
     issue_tile(1, jq0 + 1);
+    issue_tile(2, jq0 + 2);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * C::LOADS_PER_TILE) : "memory");
+    __syncthreads();
 
-    int st = 0;
+    // Software pipeline over 32-row sub-tiles: the score products of the next sub-tile are issued
+    // among the exponentials of the current one.  Tile it+1 is awaited (and tile it+3 requested,
+    // into the stage tile it-1 has left) between the two sub-tiles of tile it, so four stages.
+    // Sub-tiles wholly above the causal diagonal of a wave are not skipped: the mask zeroes them.
+    f32x16 sA, dpA, sB, dpB;
+    bf16x8 pf[2], dsf[2];
+    scores(lds, lds + C::TILE, 0, sA, dpA);
     for (int it = 0; it < ntile; ++it) {
-        // all but the most recent tile's requests have landed
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::LOADS_PER_TILE) : "memory");
-        __syncthreads();
-        {
-            const int st2 = st + 2 >= C::NST ? st + 2 - C::NST : st + 2;
-            issue_tile(st2, jq0 + it + 2);
-        }
         const int q0 = (jq0 + it) * C::BQ;
-        const unsigned char* Qt = lds + st * C::STAGE;
+        const unsigned char* Qt = lds + (it & (C::NST - 1)) * C::STAGE;
         const unsigned char* dOt = Qt + C::TILE;
         const unsigned char* St = Qt + 2 * C::TILE;
-#pragma unroll
-        for (int T = 0; T < 2; ++T) {
-            const int qs0 = q0 + 32 * T;
-            if (CAUSAL && qs0 + 31 < nw0) continue;          // every query of the sub-tile precedes every key of the wave
-            f32x16 s, dp;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) { s[e] = 0.0f; dp[e] = 0.0f; }
-#pragma unroll
-            for (int i = 0; i < C::KSTEPS; ++i) {
-                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qt + row_off[i] + T * 32 * C::ROW);
-                s = mfma_32x32x16_bf16(qa, kf[i], s);
-                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOt + row_off[i] + T * 32 * C::ROW);
-                dp = mfma_32x32x16_bf16(da, vf[i], dp);
-            }
-            // register e <-> query row qs0 + 8(e/4) + 4g + e%4 ; its (lse2, delta) pair sits at
-            // pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte
-            const bool need_mask = CAUSAL && (qs0 < nw0 + 31);
-            bf16x8 pf[2], dsf[2];
-#pragma unroll
-            for (int sh = 0; sh < 2; ++sh) {
-                u32x4 ppk, dpk;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {                // e/4 = 2sh + h
-                    const int prow = 32 * T + 8 * (2 * sh + h) + 4 * g;
-                    const f32x4 a = *reinterpret_cast<const f32x4*>(St + prow * 8);
-                    const f32x4 b = *reinterpret_cast<const f32x4*>(St + prow * 8 + 16);
-                    const float l2[4] = {a[0], a[2], b[0], b[2]};
-                    const float dl[4] = {a[1], a[3], b[1], b[3]};
-                    float p[4], ds[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const int e = 8 * sh + 4 * h + x;
-                        float pv = fast_exp2(fmaf(s[e], scale_log2, -l2[x]));
-                        if (need_mask && kvpos > qs0 + 8 * (2 * sh + h) + 4 * g + x) pv = 0.0f;
-                        p[x] = pv;
-                        ds[x] = pv * (dp[e] - dl[x]);
-                    }
-                    ppk[2 * h] = pack_bf16(p[0], p[1]);
-                    ppk[2 * h + 1] = pack_bf16(p[2], p[3]);
-                    dpk[2 * h] = pack_bf16(ds[0], ds[1]);
-                    dpk[2 * h + 1] = pack_bf16(ds[2], ds[3]);
-                }
-                pf[sh] = __builtin_bit_cast(bf16x8, ppk);
-                dsf[sh] = __builtin_bit_cast(bf16x8, dpk);
-            }
-            // dV^T += dO^T P ; dK^T += Q^T dS   (k-step c = 2T + sh: query rows 16c + 8h + 4g + [0,4))
-#pragma unroll
-            for (int sh = 0; sh < 2; ++sh) {
-                const int c = 2 * T + sh;
-#pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt) {
-                    const bf16x4 lo = ds_read_tr16(dOt + tr_lo[dt] + c * 16 * C::ROW);
-                    const bf16x4 hi = ds_read_tr16(dOt + tr_hi[dt] + c * 16 * C::ROW);
-                    dv[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf[sh], dv[dt]);
-                    const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
-                    const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
-                    dk[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7), dsf[sh], dk[dt]);
-                }
-            }
+        // the branch on the mask encloses the score products so that each side is one block of
+        // straight-line code in which they interleave with the exponentials
+        if (CAUSAL && q0 < nw0 + 31) {
+            scores(Qt, dOt, 1, sB, dpB);
+            probabilities(std::true_type{}, St, 0, q0, sA, dpA, pf, dsf);
+        } else {
+            scores(Qt, dOt, 1, sB, dpB);
+            probabilities(std::false_type{}, St, 0, q0, sA, dpA, pf, dsf);
         }
-        st = st + 1 == C::NST ? 0 : st + 1;
+        accumulate(Qt, dOt, 0, pf, dsf);
+        const bool more = it + 1 < ntile;
+        const unsigned char* Qn = lds + ((it + 1) & (C::NST - 1)) * C::STAGE;
+        if (more) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::LOADS_PER_TILE) : "memory");
+            __syncthreads();
+            issue_tile((it + 3) & (C::NST - 1), jq0 + it + 3);
+        }
+        if (CAUSAL && q0 + 32 < nw0 + 31) {
+            if (more) scores(Qn, Qn + C::TILE, 0, sA, dpA);
+            probabilities(std::true_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
+        } else if (more) {
+            scores(Qn, Qn + C::TILE, 0, sA, dpA);
+            probabilities(std::false_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
+        } else {
+            probabilities(std::false_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
+        }
+        accumulate(Qt, dOt, 1, pf, dsf);
     }
     wait_vmcnt0();
     __syncthreads();
