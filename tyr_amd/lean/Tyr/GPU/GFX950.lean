@@ -43,6 +43,17 @@ def capabilities : Capabilities := {}
 opaque flashAttnFwd {B H N D : UInt64} (q k v : @& T #[B, H, N, D]) (causal : Bool) (scale : Float)
     (stream : CudaStream) : IO (T #[B, H, N, D] × T #[B, H, N])
 
+/-- Flash-attention backward. `o` and `lse` are the results of `flashAttnFwd` for the same
+    `q k v causal scale`; `dO` is the upstream gradient. Returns `(dQ, dK, dV)`, bf16, final
+    (no per-tile partials to reduce on the host). Replaces `tkMhaH100BwdPrep2Block` +
+    `tkMhaH100Bwd2BlockPartials` (`Tyr/GPU/Kernels/MhaH100.lean:197-344`) for any `B H N`;
+    the values are autograd's for `nn.scaled_dot_product_attention`
+    (`Examples/GPU/RunMhaH100.lean:56-64`). -/
+@[extern "lean_tyr_gpu_flash_attn_bwd"]
+opaque flashAttnBwd {B H N D : UInt64} (q k v o : @& T #[B, H, N, D]) (lse : @& T #[B, H, N])
+    (dO : @& T #[B, H, N, D]) (causal : Bool) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, H, N, D] × T #[B, H, N, D] × T #[B, H, N, D])
+
 /-- GQA decode attention, one query token per sequence, split-KV with an LSE combine pass.
     `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D = 128`,
     query head `h` reads kv head `h / (Hq/Hkv)`; `numSplits = 0` lets the library choose.
