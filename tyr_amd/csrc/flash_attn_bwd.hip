@@ -408,25 +408,32 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
 
     const int jq0 = CAUSAL ? n0 / C::BQ : 0;
     const int ntile = nq - jq0;
+    const int nsub = 2 * ntile;                       // 32-row sub-tiles, numbered from the block's first tile
+    // First sub-tile with a visible (query, key) pair for this wave.  Causal: the block's first
+    // tile starts at query n0 and the wave's keys at n0 + 32w, so sub-tile w is the wave's diagonal
+    // one (the only partially masked one); earlier sub-tiles are skipped.
+    const int u0 = CAUSAL ? w : 0;
 
-    // S and dP of one 32-row sub-tile T of the tile staged at Qt / dOt
-    auto scores = [&](const unsigned char* Qt, const unsigned char* dOt, int T, f32x16& s, f32x16& dp) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) { s[e] = 0.0f; dp[e] = 0.0f; }
-        bf16x8 qa[C::KSTEPS], da[C::KSTEPS];          // all row fragments are requested up front
+    // Row fragments (lane = query row) of sub-tile T of the tile staged at Qt
+    auto read_rows = [&](const unsigned char* Qt, int T, bf16x8 (&qa)[C::KSTEPS], bf16x8 (&da)[C::KSTEPS]) {
 #pragma unroll
         for (int i = 0; i < C::KSTEPS; ++i) {
             qa[i] = *reinterpret_cast<const bf16x8*>(Qt + row_off[i] + T * 32 * C::ROW);
-            da[i] = *reinterpret_cast<const bf16x8*>(dOt + row_off[i] + T * 32 * C::ROW);
+            da[i] = *reinterpret_cast<const bf16x8*>(Qt + C::TILE + row_off[i] + T * 32 * C::ROW);
         }
+    };
+    // S = Q K_w^T and dP = dO V_w^T of one sub-tile from its row fragments
+    auto scores = [&](const bf16x8 (&qa)[C::KSTEPS], const bf16x8 (&da)[C::KSTEPS], f32x16& s, f32x16& dp) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { s[e] = 0.0f; dp[e] = 0.0f; }
 #pragma unroll
         for (int i = 0; i < C::KSTEPS; ++i) {
             s = mfma_32x32x16_bf16(qa[i], kf[i], s);
             dp = mfma_32x32x16_bf16(da[i], vf[i], dp);
         }
     };
-    // P and dS of that sub-tile as column operands.  Register e <-> query row qs0 + 8(e/4) + 4g +
-    // e%4; its (lse2, delta) pair sits at pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte.
+    // P and dS of a sub-tile as column operands.  Register e <-> query row qs0 + 8(e/4) + 4g + e%4;
+    // its (lse2, delta) pair sits at pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte.
     auto probabilities = [&](auto masked, const unsigned char* St, int T, int qs0, const f32x16& s,
                              const f32x16& dp, bf16x8 (&pf)[2], bf16x8 (&dsf)[2]) {
         constexpr bool need_mask = decltype(masked)::value;
@@ -443,7 +450,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
                 float p[4], ds[4];
 #pragma unroll
                 for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
-                if (need_mask) {                         // only tiles that touch the diagonal
+                if (need_mask) {
 #pragma unroll
                     for (int x = 0; x < 4; ++x)
                         if (kvpos > qs0 + 8 * (2 * sh + h) + 4 * g + x) p[x] = 0.0f;
@@ -459,21 +466,51 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             dsf[sh] = __builtin_bit_cast(bf16x8, dpk);
         }
     };
-    // dV^T += dO^T P ; dK^T += Q^T dS   (k-step c = 2T + sh: query rows 16c + 8h + 4g + [0,4))
-    auto accumulate = [&](const unsigned char* Qt, const unsigned char* dOt, int T, const bf16x8 (&pf)[2],
-                          const bf16x8 (&dsf)[2]) {
+    // Transposed fragments of k-step c = 2T + sh (query rows 16c + 8h + 4g + [0,4)) of dO and Q
+    auto read_transposed = [&](const unsigned char* Qt, int c, bf16x8 (&dot)[C::DT], bf16x8 (&qt)[C::DT]) {
 #pragma unroll
-        for (int sh = 0; sh < 2; ++sh) {
-            const int c = 2 * T + sh;
+        for (int dt = 0; dt < C::DT; ++dt) {
+            const bf16x4 lo = ds_read_tr16(Qt + C::TILE + tr_lo[dt] + c * 16 * C::ROW);
+            const bf16x4 hi = ds_read_tr16(Qt + C::TILE + tr_hi[dt] + c * 16 * C::ROW);
+            dot[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
+            const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
+            qt[dt] = __builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+
+    bf16x8 rq[C::KSTEPS], rd[C::KSTEPS];              // row fragments of the next sub-tile, read one step ahead
+    auto stage_of = [&](int tile) { return lds + (tile & (C::NST - 1)) * C::STAGE; };
+    // One step of the software pipeline on sub-tile u (scores in sc / dpc): the score products of
+    // sub-tile u+1 (row fragments already in rq / rd) are issued among the exponentials of u, the
+    // row fragments of u+2 are requested under the dV / dK products of u.  With one wave per SIMD
+    // nothing else hides LDS latency, so every fragment is requested a phase before its use.
+    // Past the last sub-tile the "next" work is redone on the last tile and dropped.
+    auto step = [&](auto masked, auto first, int u, f32x16& sc, f32x16& dpc, f32x16& sn, f32x16& dpn) {
+        const int t = u >> 1, T = u & 1;
+        const unsigned char* Qt = stage_of(t);
+        const int u1 = u + 1 < nsub ? u + 1 : u, u2 = u + 2 < nsub ? u + 2 : u;
+        if (decltype(first)::value) {                 // the wave's first sub-tile: nothing was prepared
+            read_rows(Qt, T, rq, rd);
+            scores(rq, rd, sc, dpc);
+            read_rows(stage_of(u1 >> 1), u1 & 1, rq, rd);
+        }
+        bf16x8 dot0[C::DT], qt0[C::DT], dot1[C::DT], qt1[C::DT];
+        read_transposed(Qt, 2 * T, dot0, qt0);
+        scores(rq, rd, sn, dpn);
+        bf16x8 pf[2], dsf[2];
+        probabilities(masked, Qt + 2 * C::TILE, T, (jq0 + t) * C::BQ + 32 * T, sc, dpc, pf, dsf);
+        read_transposed(Qt, 2 * T + 1, dot1, qt1);
+        read_rows(stage_of(u2 >> 1), u2 & 1, rq, rd);
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt) {
-                const bf16x4 lo = ds_read_tr16(dOt + tr_lo[dt] + c * 16 * C::ROW);
-                const bf16x4 hi = ds_read_tr16(dOt + tr_hi[dt] + c * 16 * C::ROW);
-                dv[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf[sh], dv[dt]);
-                const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
-                const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
-                dk[dt] = mfma_32x32x16_bf16(__builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7), dsf[sh], dk[dt]);
-            }
+        for (int dt = 0; dt < C::DT; ++dt) {
+            dv[dt] = mfma_32x32x16_bf16(dot0[dt], pf[0], dv[dt]);
+            dk[dt] = mfma_32x32x16_bf16(qt0[dt], dsf[0], dk[dt]);
+        }
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+            dv[dt] = mfma_32x32x16_bf16(dot1[dt], pf[1], dv[dt]);
+            dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf[1], dk[dt]);
         }
     };
 
@@ -485,45 +522,28 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * C::LOADS_PER_TILE) : "memory");
     __syncthreads();
 
-    // Software pipeline over 32-row sub-tiles: the score products of the next sub-tile are issued
-    // among the exponentials of the current one.  Tile it+1 is awaited (and tile it+3 requested,
-    // into the stage tile it-1 has left) between the two sub-tiles of tile it, so four stages.
-    // Sub-tiles wholly above the causal diagonal of a wave are not skipped: the mask zeroes them.
-    f32x16 sA, dpA, sB, dpB;
-    bf16x8 pf[2], dsf[2];
-    scores(lds, lds + C::TILE, 0, sA, dpA);
-    for (int it = 0; it < ntile; ++it) {
-        const int q0 = (jq0 + it) * C::BQ;
-        const unsigned char* Qt = lds + (it & (C::NST - 1)) * C::STAGE;
-        const unsigned char* dOt = Qt + C::TILE;
-        const unsigned char* St = Qt + 2 * C::TILE;
-        // the branch on the mask encloses the score products so that each side is one block of
-        // straight-line code in which they interleave with the exponentials
-        if (CAUSAL && q0 < nw0 + 31) {
-            scores(Qt, dOt, 1, sB, dpB);
-            probabilities(std::true_type{}, St, 0, q0, sA, dpA, pf, dsf);
-        } else {
-            scores(Qt, dOt, 1, sB, dpB);
-            probabilities(std::false_type{}, St, 0, q0, sA, dpA, pf, dsf);
-        }
-        accumulate(Qt, dOt, 0, pf, dsf);
-        const bool more = it + 1 < ntile;
-        const unsigned char* Qn = lds + ((it + 1) & (C::NST - 1)) * C::STAGE;
-        if (more) {
+    // Tile t+1 is awaited, and tile t+3 requested into the stage tile t-1 has left, before the
+    // first sub-tile of tile t (whose steps already read fragments of tile t+1): four stages.
+    auto tile_boundary = [&](int u) {
+        if (!(u & 1) && (u >> 1) + 1 < ntile) {
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::LOADS_PER_TILE) : "memory");
             __syncthreads();
-            issue_tile((it + 3) & (C::NST - 1), jq0 + it + 3);
+            issue_tile(((u >> 1) + 3) & (C::NST - 1), jq0 + (u >> 1) + 3);
         }
-        if (CAUSAL && q0 + 32 < nw0 + 31) {
-            if (more) scores(Qn, Qn + C::TILE, 0, sA, dpA);
-            probabilities(std::true_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
-        } else if (more) {
-            scores(Qn, Qn + C::TILE, 0, sA, dpA);
-            probabilities(std::false_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
-        } else {
-            probabilities(std::false_type{}, St, 1, q0 + 32, sB, dpB, pf, dsf);
-        }
-        accumulate(Qt, dOt, 1, pf, dsf);
+    };
+    f32x16 sc, dpc, sn, dpn;
+    int u = 0;
+    for (; u < u0 && u < nsub; ++u) tile_boundary(u);           // sub-tiles above the wave's diagonal
+    if (u < nsub) {
+        tile_boundary(u);
+        step(std::integral_constant<bool, CAUSAL>{}, std::true_type{}, u, sc, dpc, sn, dpn);
+        ++u;
+    }
+    for (; u < nsub; ++u) {
+        sc = sn;
+        dpc = dpn;
+        tile_boundary(u);
+        step(std::false_type{}, std::false_type{}, u, sc, dpc, sn, dpn);
     }
     wait_vmcnt0();
     __syncthreads();
