@@ -414,12 +414,44 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     // one (the only partially masked one); earlier sub-tiles are skipped.
     const int u0 = CAUSAL ? w : 0;
 
-    // Row fragments (lane = query row) of sub-tile T of the tile staged at Qt
-    auto read_rows = [&](const unsigned char* Qt, int T, bf16x8 (&qa)[C::KSTEPS], bf16x8 (&da)[C::KSTEPS]) {
+    // LDS addresses.  Inside the pipeline the stage and the sub-tile of every access are
+    // compile-time constants, so an address is a per-lane base register plus an immediate; the
+    // immediate field holds 16 bits, hence a second set of bases for stages 2 and 3.
+    // The bases are made opaque to the compiler, which would otherwise recompute each of them
+    // (LDS symbol + offset) next to every use.
+    typedef __attribute__((address_space(3))) const unsigned char* lds_cptr;
+    auto opaque = [&](int off) {
+        uint32_t a = lds_base + (uint32_t)off;
+        asm volatile("" : "+v"(a));
+        return (lds_cptr)(uintptr_t)a;
+    };
+    lds_cptr rowp[2][C::KSTEPS], trlo[2][C::DT], trhi[2][C::DT], statp[2];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) rowp[hh][i] = opaque(row_off[i] + hh * 2 * C::STAGE);
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt) {
+            trlo[hh][dt] = opaque(tr_lo[dt] + hh * 2 * C::STAGE);
+            trhi[hh][dt] = opaque(tr_hi[dt] + hh * 2 * C::STAGE);
+        }
+        statp[hh] = opaque(2 * C::TILE + 32 * g + hh * 2 * C::STAGE);
+    }
+    auto tr16 = [](lds_cptr p) {
+        typedef __attribute__((ext_vector_type(4))) short s16x4;
+        return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p)));
+    };
+#define TYR_STG(stg) constexpr int STG = decltype(stg)::value; constexpr int SOFF = (STG & 1) * C::STAGE
+
+    // Row fragments (lane = query row) of sub-tile T of the tile in stage STG
+    auto read_rows = [&](auto stg, auto sub, bf16x8 (&qa)[C::KSTEPS], bf16x8 (&da)[C::KSTEPS]) {
+        TYR_STG(stg);
+        constexpr int T = decltype(sub)::value;
 #pragma unroll
         for (int i = 0; i < C::KSTEPS; ++i) {
-            qa[i] = *reinterpret_cast<const bf16x8*>(Qt + row_off[i] + T * 32 * C::ROW);
-            da[i] = *reinterpret_cast<const bf16x8*>(Qt + C::TILE + row_off[i] + T * 32 * C::ROW);
+            lds_cptr p = rowp[STG >> 1][i] + SOFF + T * 32 * C::ROW;
+            qa[i] = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(p);
+            da[i] = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(p + C::TILE);
         }
     };
     // S = Q K_w^T and dP = dO V_w^T of one sub-tile from its row fragments
@@ -434,17 +466,26 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     };
     // P and dS of a sub-tile as column operands.  Register e <-> query row qs0 + 8(e/4) + 4g + e%4;
     // its (lse2, delta) pair sits at pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte.
-    auto probabilities = [&](auto masked, const unsigned char* St, int T, int qs0, const f32x16& s,
-                             const f32x16& dp, bf16x8 (&pf)[2], bf16x8 (&dsf)[2]) {
+    auto read_pairs = [&](auto stg, auto sub, f32x4 (&st)[8]) {
+        TYR_STG(stg);
+        constexpr int T = decltype(sub)::value;
+        lds_cptr St = statp[STG >> 1] + SOFF + 32 * T * 8;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {                    // k = e/4
+            st[2 * k] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * k * 8);
+            st[2 * k + 1] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * k * 8 + 16);
+        }
+    };
+    auto probabilities = [&](auto masked, const f32x4 (&st)[8], int qs0, const f32x16& s, const f32x16& dp,
+                             bf16x8 (&pf)[2], bf16x8 (&dsf)[2]) {
         constexpr bool need_mask = decltype(masked)::value;
 #pragma unroll
         for (int sh = 0; sh < 2; ++sh) {
             u32x4 ppk, dpk;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {                // e/4 = 2sh + h
-                const int prow = 32 * T + 8 * (2 * sh + h) + 4 * g;
-                const f32x4 a = *reinterpret_cast<const f32x4*>(St + prow * 8);
-                const f32x4 b = *reinterpret_cast<const f32x4*>(St + prow * 8 + 16);
+                const f32x4 a = st[2 * (2 * sh + h)];
+                const f32x4 b = st[2 * (2 * sh + h) + 1];
                 const float l2[4] = {a[0], a[2], b[0], b[2]};
                 const float dl[4] = {a[1], a[3], b[1], b[3]};
                 float p[4], ds[4];
@@ -467,41 +508,48 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         }
     };
     // Transposed fragments of k-step c = 2T + sh (query rows 16c + 8h + 4g + [0,4)) of dO and Q
-    auto read_transposed = [&](const unsigned char* Qt, int c, bf16x8 (&dot)[C::DT], bf16x8 (&qt)[C::DT]) {
+    auto read_transposed = [&](auto stg, int c, bf16x8 (&dot)[C::DT], bf16x8 (&qt)[C::DT]) {
+        TYR_STG(stg);
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
-            const bf16x4 lo = ds_read_tr16(Qt + C::TILE + tr_lo[dt] + c * 16 * C::ROW);
-            const bf16x4 hi = ds_read_tr16(Qt + C::TILE + tr_hi[dt] + c * 16 * C::ROW);
+            lds_cptr pl = trlo[STG >> 1][dt] + SOFF + c * 16 * C::ROW;
+            lds_cptr ph = trhi[STG >> 1][dt] + SOFF + c * 16 * C::ROW;
+            const bf16x4 lo = tr16(pl + C::TILE);
+            const bf16x4 hi = tr16(ph + C::TILE);
             dot[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            const bf16x4 ql = ds_read_tr16(Qt + tr_lo[dt] + c * 16 * C::ROW);
-            const bf16x4 qh = ds_read_tr16(Qt + tr_hi[dt] + c * 16 * C::ROW);
+            const bf16x4 ql = tr16(pl);
+            const bf16x4 qh = tr16(ph);
             qt[dt] = __builtin_shufflevector(ql, qh, 0, 1, 2, 3, 4, 5, 6, 7);
         }
     };
 
     bf16x8 rq[C::KSTEPS], rd[C::KSTEPS];              // row fragments of the next sub-tile, read one step ahead
-    auto stage_of = [&](int tile) { return lds + (tile & (C::NST - 1)) * C::STAGE; };
-    // One step of the software pipeline on sub-tile u (scores in sc / dpc): the score products of
-    // sub-tile u+1 (row fragments already in rq / rd) are issued among the exponentials of u, the
-    // row fragments of u+2 are requested under the dV / dK products of u.  With one wave per SIMD
-    // nothing else hides LDS latency, so every fragment is requested a phase before its use.
-    // Past the last sub-tile the "next" work is redone on the last tile and dropped.
-    auto step = [&](auto masked, auto first, int u, f32x16& sc, f32x16& dpc, f32x16& sn, f32x16& dpn) {
-        const int t = u >> 1, T = u & 1;
-        const unsigned char* Qt = stage_of(t);
-        const int u1 = u + 1 < nsub ? u + 1 : u, u2 = u + 2 < nsub ? u + 2 : u;
+    // One step of the software pipeline on sub-tile u = 2t + T, tile t in stage STG (scores in sc /
+    // dpc): the score products of sub-tile u+1 (row fragments already in rq / rd) are issued among
+    // the exponentials of u, the row fragments of u+2 are requested under the dV / dK products of u.
+    // With one wave per SIMD nothing else hides LDS latency and every instruction of the wave costs
+    // issue time, so fragments are requested a phase ahead and addresses cost no instructions.
+    // Past the last sub-tile the "next" reads hit a stage without live data; their results are dropped.
+    auto step = [&](auto masked, auto first, auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc, f32x16& sn,
+                    f32x16& dpn) {
+        constexpr int STG = decltype(stg)::value, T = decltype(sub)::value;
+        using Stg1 = std::integral_constant<int, T == 0 ? STG : ((STG + 1) & 3)>;     // stage of u+1
+        using Sub1 = std::integral_constant<int, 1 - T>;
+        using Stg2 = std::integral_constant<int, (STG + 1) & 3>;                        // stage of u+2
         if (decltype(first)::value) {                 // the wave's first sub-tile: nothing was prepared
-            read_rows(Qt, T, rq, rd);
+            read_rows(stg, sub, rq, rd);
             scores(rq, rd, sc, dpc);
-            read_rows(stage_of(u1 >> 1), u1 & 1, rq, rd);
+            read_rows(Stg1{}, Sub1{}, rq, rd);
         }
         bf16x8 dot0[C::DT], qt0[C::DT], dot1[C::DT], qt1[C::DT];
-        read_transposed(Qt, 2 * T, dot0, qt0);
+        read_transposed(stg, 2 * T, dot0, qt0);
+        f32x4 st[8];
+        read_pairs(stg, sub, st);
         scores(rq, rd, sn, dpn);
         bf16x8 pf[2], dsf[2];
-        probabilities(masked, Qt + 2 * C::TILE, T, (jq0 + t) * C::BQ + 32 * T, sc, dpc, pf, dsf);
-        read_transposed(Qt, 2 * T + 1, dot1, qt1);
-        read_rows(stage_of(u2 >> 1), u2 & 1, rq, rd);
+        probabilities(masked, st, qs0, sc, dpc, pf, dsf);
+        read_transposed(stg, 2 * T + 1, dot1, qt1);
+        read_rows(Stg2{}, sub, rq, rd);
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
             dv[dt] = mfma_32x32x16_bf16(dot0[dt], pf[0], dv[dt]);
@@ -513,6 +561,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf[1], dk[dt]);
         }
     };
+#undef TYR_STG
 
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(kf[i]); pin_registers(vf[i]); }
@@ -531,20 +580,48 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             issue_tile(((u >> 1) + 3) & (C::NST - 1), jq0 + (u >> 1) + 3);
         }
     };
-    f32x16 sc, dpc, sn, dpn;
+    using std::integral_constant;
+    using MaskedT = integral_constant<bool, CAUSAL>;
+    const int qbase = jq0 * C::BQ;
+    // Scores ping-pong between two register sets by the parity of u (no copies).
+    f32x16 sA, dpA, sB, dpB;
     int u = 0;
     for (; u < u0 && u < nsub; ++u) tile_boundary(u);           // sub-tiles above the wave's diagonal
     if (u < nsub) {
         tile_boundary(u);
-        step(std::integral_constant<bool, CAUSAL>{}, std::true_type{}, u, sc, dpc, sn, dpn);
+        // u = u0 < 4: stage u0 / 2, sub-tile u0 % 2
+        switch (u) {
+            case 0:  step(MaskedT{}, std::true_type{}, integral_constant<int, 0>{}, integral_constant<int, 0>{}, qbase, sA, dpA, sB, dpB); break;
+            case 1:  step(MaskedT{}, std::true_type{}, integral_constant<int, 0>{}, integral_constant<int, 1>{}, qbase + 32, sB, dpB, sA, dpA); break;
+            case 2:  step(MaskedT{}, std::true_type{}, integral_constant<int, 1>{}, integral_constant<int, 0>{}, qbase + 64, sA, dpA, sB, dpB); break;
+            default: step(MaskedT{}, std::true_type{}, integral_constant<int, 1>{}, integral_constant<int, 1>{}, qbase + 96, sB, dpB, sA, dpA); break;
+        }
         ++u;
     }
-    for (; u < nsub; ++u) {
-        sc = sn;
-        dpc = dpn;
-        tile_boundary(u);
-        step(std::false_type{}, std::false_type{}, u, sc, dpc, sn, dpn);
+    // steady state, unrolled over the 8 (stage, sub-tile) combinations; entered at u % 8
+#define TYR_STEP(K, CS, CD, NS, ND)                                                                          \
+    case K:                                                                                                  \
+        if (u >= nsub) goto pipeline_done;                                                                   \
+        tile_boundary(u);                                                                                    \
+        step(std::false_type{}, std::false_type{}, integral_constant<int, (K) / 2>{},                        \
+             integral_constant<int, (K) % 2>{}, qbase + 32 * u, CS, CD, NS, ND);                             \
+        ++u;                                                                                                 \
+        [[fallthrough]];
+    for (;;) {
+        switch (u & 7) {
+            TYR_STEP(0, sA, dpA, sB, dpB)
+            TYR_STEP(1, sB, dpB, sA, dpA)
+            TYR_STEP(2, sA, dpA, sB, dpB)
+            TYR_STEP(3, sB, dpB, sA, dpA)
+            TYR_STEP(4, sA, dpA, sB, dpB)
+            TYR_STEP(5, sB, dpB, sA, dpA)
+            TYR_STEP(6, sA, dpA, sB, dpB)
+            TYR_STEP(7, sB, dpB, sA, dpA)
+            default: break;
+        }
     }
+pipeline_done:
+#undef TYR_STEP
     wait_vmcnt0();
     __syncthreads();
 
