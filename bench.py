@@ -13,6 +13,7 @@ FLOP / byte conventions (algorithmic work, fixed per configuration):
   attn_fwd_causal : 4*B*H*N^2*D / 2 FLOP (two GEMMs, causal half)           -> MFMA bf16 2.5 PFLOP/s
   attn_bwd_causal : 10*B*H*N^2*D / 2 FLOP (five GEMMs, causal half)         -> MFMA bf16 2.5 PFLOP/s
   gqa_decode      : bytes of K + V + Q + O                                   -> HBM 8 TB/s
+  decode_step, rope_fwd, layernorm_residual, copy_kernel : bytes read + written      -> HBM 8 TB/s
   gemm_bf16       : 2*M*N*K FLOP                                             -> MFMA bf16 2.5 PFLOP/s
   gemm_fp8        : 2*M*N*K FLOP                                             -> MFMA fp8 5.0 PFLOP/s
 Kernel durations are measured with HIP events on the stream the kernels are launched on.
@@ -248,6 +249,120 @@ def wl_gemm_fp8(torch, tyr, steps, warmup, cpu):
     return res
 
 
+def _hbm_result(metric, workload, kernel, nbytes, ms, wall, dtype, extra=None):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    cfg = {"workload": workload, "bytes_convention": f"{nbytes:,} B read + written per launch"}
+    if extra:
+        cfg.update(extra)
+    return {"metric": metric, "value": gbs, "unit": "GB/s", "ms_per_step": ms, "wall_ms_per_step": wall, "dtype": dtype,
+            "config": cfg,
+            "roofline": {"bound": "hbm", "kernel": kernel, "achieved": gbs, "peak": PEAK["hbm"], "unit": "GB/s",
+                         "frac": gbs / PEAK["hbm"], "traffic": TRAFFIC.get(kernel)}}
+
+
+def _cpu_time(fn, budget=6.0, max_reps=30):
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 2 or (time.perf_counter() - t0 < budget and reps < max_reps):
+        fn()
+        reps += 1
+    return (time.perf_counter() - t0) / reps, reps
+
+
+def wl_rope(torch, tyr, steps, warmup, cpu):
+    from oracle import libtorch_path as lt
+    B, S, H, D = 16, 4096, 16, 128
+    torch.manual_seed(0)
+    xs = [torch.randn(B, S, H, D, device="cuda").to(torch.bfloat16) for _ in range(3)]   # 268 MB each, rotated
+    cos, sin = (t.cuda() for t in lt.compute_rotary_freqs(S, D))
+    it = [0]
+
+    def fn():
+        it[0] += 1
+        return tyr.rope_fwd(xs[it[0] % 3], cos, sin)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    nbytes = 2 * B * S * H * D * 2 + 2 * S * (D // 2) * 4
+    res = _hbm_result("rotary GB/s", "rotary embedding, bf16 [16,4096,16,128], cos/sin f32 [4096,64]",
+                      "rope_kernel<bf16>", nbytes, ms, wall, "f32 arithmetic on bf16 data")
+    if cpu:
+        xc = xs[0][:1].cpu()
+        dt, reps = _cpu_time(lambda: lt.apply_rotary_emb(xc, cos.cpu(), sin.cpu()))
+        res["cpu_baseline"] = {"value": nbytes / B / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU slice/mul/sub/cat sequence on 1 of 16 batch entries, {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_layernorm(torch, tyr, steps, warmup, cpu):
+    from oracle import libtorch_path as lt
+    rows, d = 65536, 1024
+    torch.manual_seed(0)
+    xs = [(torch.rand(rows, d, device="cuda").to(torch.bfloat16), torch.rand(rows, d, device="cuda").to(torch.bfloat16))
+          for _ in range(3)]
+    w, b = torch.rand(d, device="cuda").to(torch.bfloat16), torch.rand(d, device="cuda").to(torch.bfloat16)
+    it = [0]
+
+    def fn():
+        it[0] += 1
+        x, r = xs[it[0] % 3]
+        return tyr.layernorm_residual(x, r, w, b, 1e-5)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    nbytes = 4 * rows * d * 2 + 2 * d * 2
+    res = _hbm_result("layernorm GB/s", "fused residual + LayerNorm, bf16, 65536 rows of 1024",
+                      "layernorm_residual_kernel<2>", nbytes, ms, wall, "f32 arithmetic on bf16 data")
+    if cpu:
+        xc, rc = (t[:4096].cpu() for t in xs[0])
+        dt, reps = _cpu_time(lambda: lt.layer_norm_residual(xc, rc, w.cpu(), b.cpu(), 1e-5))
+        res["cpu_baseline"] = {"value": nbytes / 16 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU add + layer_norm on 4096 of 65536 rows, {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_copy_kernel(torch, tyr, steps, warmup, cpu):
+    n = 1 << 30
+    srcs = [torch.empty(n, dtype=torch.uint8, device="cuda").random_() for _ in range(2)]
+    it = [0]
+
+    def fn():
+        it[0] += 1
+        return tyr.copy(srcs[it[0] % 2])
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    res = _hbm_result("copy GB/s", "device copy kernel, 1 GiB", "copy_kernel", 2 * n, ms, wall, "u8")
+    if cpu:
+        sc = srcs[0][: n // 8].cpu()
+        dt, reps = _cpu_time(lambda: sc.clone())
+        res["cpu_baseline"] = {"value": 2 * (n // 8) / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU clone of 128 MiB, {reps} reps, {dt * 1e3:.0f} ms each"}
+    return res
+
+
+def wl_decode_step(torch, tyr, steps, warmup, cpu):
+    """The decode step's cache update followed by attention over the cache (forwardStep order)."""
+    from oracle import libtorch_path as lt
+    B, Hq, Hkv, L, D = 32, 32, 8, 8192, 128
+    torch.manual_seed(1)
+    q = torch.randn(B, Hq, 1, D, device="cuda").to(torch.bfloat16)
+    kn, vn = (torch.randn(B, Hkv, 1, D, device="cuda").to(torch.bfloat16) for _ in range(2))
+    caches = [(torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16),
+               torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16)) for _ in range(4)]
+    cos_t, sin_t = lt.compute_rotary_freqs(L, D)
+    cos, sin = cos_t[L - 1:].contiguous().cuda(), sin_t[L - 1:].contiguous().cuda()
+    sc = 1.0 / math.sqrt(D)
+    it = [0]
+
+    def fn():
+        k, v = caches[it[0] % len(caches)]
+        it[0] += 1
+        qr = tyr.decode_rope_append(q, kn, vn, cos, sin, k, v, L - 1)
+        return tyr.gqa_decode(qr, k, v, scale=sc, kv_len=L)
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    nbytes = 2 * B * Hkv * L * D * 2 + 2 * B * Hq * D * 2
+    res = _hbm_result("decode step GB/s", "decode step: rotate q/k + append k/v to the cache (position 8191) + GQA decode "
+                      "attention over 8192 cached rows, bf16, batch 32, 32 q heads, 8 kv heads, D=128",
+                      "decode_rope_append_kernel + gqa_decode_split_kernel<8>", nbytes, ms, wall, "bf16",
+                      {"bytes_convention": "bytes of the attention pass (K + V + Q + O); the append moves 0.4 MB more"})
+    return res
+
+
 def wl_copy(torch, tyr, steps, warmup, cpu):
     """Counter calibration only: a plain device copy of exactly 1 GiB (reads 2^30 B, writes 2^30 B)."""
     n = 1 << 30
@@ -261,7 +376,9 @@ def wl_copy(torch, tyr, steps, warmup, cpu):
                          "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": 2.0 * n}}
 
 
-WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16, "gemm_fp8": wl_gemm_fp8}
+WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16,
+             "gemm_fp8": wl_gemm_fp8, "decode_step": wl_decode_step, "rope_fwd": wl_rope, "layernorm_residual": wl_layernorm,
+             "copy_kernel": wl_copy_kernel}
 CALIBRATION = {"copy_1gib": wl_copy}
 
 

@@ -132,6 +132,69 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Decode step: rotary embedding of the new q and k, append of k and v to the cache.
+ *
+ * Fuses what `QwenAttention.forwardStep` does between the projections and the
+ * attention call (Tyr/Model/Qwen/Attention.lean:172-196): `rotary.applyRotaryEmb`
+ * on the single-token q and k (cc/src/tyr.cpp:3837-3873) and `data.sliceScatter`
+ * of k and v into row `pos` of the preallocated cache.  tyr_hip_gqa_decode with
+ * L = pos + 1 and the same kv_stride then reads the cache in place.
+ *
+ *   q          : bf16 [B, Hq, D]   (the [B,1,Hq,D] projection output; same bytes as [B,Hq,1,D])
+ *   k_new,v_new: bf16 [B, Hkv, D]
+ *   cos, sin   : f32 [D/2], the row of the rotary table for position `pos`
+ *   q_out      : bf16 [B, Hq, D] (rotated q; may alias q)
+ *   k_cache, v_cache : bf16 [B, Hkv, kv_stride, D]; row `pos` of every (b, kv head) is written
+ * Supported: D % 16 == 0; pos < kv_stride.
+ */
+int tyr_hip_decode_rope_append(const void* q, const void* k_new, const void* v_new,
+                               const float* cos, const float* sin, void* q_out,
+                               void* k_cache, void* v_cache,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t D,
+                               uint64_t kv_stride, uint64_t pos, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Rotary embedding (prefill form).
+ *
+ * GPU twin of `lean_torch_apply_rotary_emb` (cc/src/tyr.cpp:3837-3873; Lean decl
+ * Tyr/Torch.lean:1044) and replacement of the DSL kernel `rotaryFwd`
+ * (Tyr/GPU/Kernels/Rotary.lean:13-66, one f32 64x64 tile) for any shape:
+ * x = [x1 | x2] split in halves along D; y1 = x1 cos - x2 sin; y2 = x1 sin + x2 cos.
+ *
+ *   x, y     : [B, S, H, D], f32 (dtype = TYR_HIP_F32) or bf16 (TYR_HIP_BF16); y may alias x
+ *   cos, sin : f32 [S, D/2]
+ * Supported: D % 8 == 0 (f32) / D % 16 == 0 (bf16).
+ */
+enum tyr_hip_dtype { TYR_HIP_F32 = 0, TYR_HIP_BF16 = 1 };
+int tyr_hip_rope_fwd(const void* x, const float* cos, const float* sin, void* y,
+                     uint64_t B, uint64_t S, uint64_t H, uint64_t D, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Fused residual add + LayerNorm.
+ *
+ * Replaces the DSL kernel `tkFusedLayerNormResidual1024`
+ * (Tyr/GPU/Kernels/FusedLayerNorm.lean:28-140; runner Examples/GPU/RunLayerNorm.lean:60-75)
+ * for any row count and any d_model % 8 == 0 up to 8192:
+ *   out_resid = bf16(x + residual)
+ *   out       = bf16((out_resid - mean) * rsqrt(var + eps) * weight + bias)
+ * with mean / var over the whole row of the rounded out_resid, in f32.
+ *
+ *   x, residual, out, out_resid : bf16 [rows, d_model]      weight, bias : bf16 [d_model]
+ */
+int tyr_hip_layernorm_residual(const void* x, const void* residual, const void* weight,
+                               const void* bias, void* out, void* out_resid,
+                               uint64_t rows, uint64_t d_model, float eps, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Device-to-device copy kernel.
+ *
+ * Replaces the DSL kernel `copy64x64` (Tyr/GPU/Kernels/Copy.lean:16-27; runner
+ * Examples/GPU/RunCopy.lean) for any byte count.  src and dst must be 16-byte
+ * aligned and must not overlap.
+ */
+int tyr_hip_copy(const void* src, void* dst, size_t bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
  * bf16 GEMM, f32 accumulation, bf16 output:  C = A B  (trans_b = 0, B is [K, N])
  *                                            C = A B^T (trans_b = 1, B is [N, K]).
  *

@@ -56,6 +56,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_gemm_bf16.restype = None
         L.oracle_gemm_fp8.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, f32, ci]
         L.oracle_gemm_fp8.restype = None
+        L.oracle_rope.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ci]
+        L.oracle_rope.restype = None
+        L.oracle_layernorm_residual.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, f64]
+        L.oracle_layernorm_residual.restype = None
         L.oracle_e4m3_decode.argtypes = [ctypes.c_uint8]
         L.oracle_e4m3_decode.restype = f32
         L.oracle_e4m3_encode.argtypes = [f32]
@@ -174,6 +178,28 @@ def gemm_fp8(aq, bq, scale_a: float, scale_b: float, trans_b: bool = False):
     lib().oracle_gemm_fp8(_p(aq), _p(bq), _p(c), _p(cf), M, N, K, float(scale_a), float(scale_b),
                           int(trans_b))
     return c, cf
+
+
+def rope(x, cos, sin):
+    """Rotary embedding.  x float32 or uint16 (bf16 bits) [B,S,H,D]; cos, sin float32 [S,D/2] -> same dtype as x."""
+    is_bf16 = x.dtype == np.uint16
+    x = _chk(x, np.uint16 if is_bf16 else np.float32, "x")
+    cos, sin = _chk(cos, np.float32, "cos"), _chk(sin, np.float32, "sin")
+    B, S, H, D = x.shape
+    y = np.empty_like(x)
+    lib().oracle_rope(_p(x), _p(cos), _p(sin), _p(y), B, S, H, D, int(is_bf16))
+    return y
+
+
+def layernorm_residual(x, residual, weight, bias, eps: float = 1e-5):
+    """Fused residual + LayerNorm.  uint16 (bf16 bits): x, residual [rows,d]; weight, bias [d] -> (out, out_resid)."""
+    x, residual = _chk(x, np.uint16, "x"), _chk(residual, np.uint16, "residual")
+    weight, bias = _chk(weight, np.uint16, "weight"), _chk(bias, np.uint16, "bias")
+    rows, d = x.shape
+    out, out_resid = np.empty_like(x), np.empty_like(x)
+    lib().oracle_layernorm_residual(_p(x), _p(residual), _p(weight), _p(bias), _p(out), _p(out_resid), rows, d,
+                                    float(eps))
+    return out, out_resid
 
 
 def num_threads() -> int:

@@ -60,6 +60,41 @@ def sdpa_gqa_qkv(q, k, v, is_causal: bool = False, enable_gqa: bool = True, drop
     return F.scaled_dot_product_attention(q, k, v, None, dropout_p, is_causal)
 
 
+def compute_rotary_freqs(seq_len: int, head_dim: int, base: float = 10000.0):
+    """(cos, sin) f32 [seq_len, head_dim/2] -- the call sequence of compute_rotary_freqs_impl."""
+    channel_range = torch.arange(0, head_dim, 2, dtype=torch.float32)
+    inv_freq = 1.0 / torch.pow(base, channel_range / float(head_dim))
+    t = torch.arange(seq_len, dtype=torch.float32)
+    freqs = torch.outer(t, inv_freq)
+    return freqs.cos(), freqs.sin()
+
+
+def apply_rotary_emb(x, cos, sin):
+    """x [B,S,H,D]; cos, sin [S,D/2] -- the call sequence of lean_torch_apply_rotary_emb."""
+    d = x.size(3) // 2
+    x1, x2 = x[..., :d], x[..., d:2 * d]
+    cos_b, sin_b = cos.unsqueeze(0).unsqueeze(2), sin.unsqueeze(0).unsqueeze(2)
+    y1 = x1 * cos_b - x2 * sin_b
+    y2 = x1 * sin_b + x2 * cos_b
+    return torch.cat([y1, y2], 3).to(x.dtype)
+
+
+def layer_norm_residual(x, residual, weight, bias, eps: float = 1e-5):
+    """(out, out_resid) as the reference's layernorm runner computes its expected values."""
+    resid = x + residual
+    return F.layer_norm(resid, (resid.shape[-1],), weight, bias, eps), resid
+
+
+def decode_step_cache_update(q, k_new, v_new, cos, sin, k_cache, v_cache, pos: int):
+    """forwardStep's RoPE + cache write: q [B,1,Hq,D], k_new / v_new [B,1,Hkv,D], cos / sin [1,D/2],
+    caches [B,Hkv,maxLen,D] -> (q_rot [B,Hq,1,D], k_cache', v_cache')."""
+    q_rot = apply_rotary_emb(q, cos, sin).transpose(1, 2)
+    k_rot = apply_rotary_emb(k_new, cos, sin).transpose(1, 2)
+    k2 = torch.slice_scatter(k_cache, k_rot, 2, pos, pos + 1)
+    v2 = torch.slice_scatter(v_cache, v_new.transpose(1, 2), 2, pos, pos + 1)
+    return q_rot, k2, v2
+
+
 def mm(a, b):
     return torch.mm(a, b)
 

@@ -32,6 +32,12 @@
  *   oracle_gemm_fp8         Tyr/GPU/Kernels/PrecisionGemm.lean:97-115,178-189 and
  *                           Tyr/GPU/Kernels/GemmCommon.lean:135-144 (scalar scale in
  *                           the f32 epilogue, bf16 out).
+ *   oracle_rope             cc/src/tyr.cpp:3837-3873 (lean_torch_apply_rotary_emb: halves
+ *                           split, y1 = x1 cos - x2 sin, y2 = x1 sin + x2 cos, f32
+ *                           arithmetic, result in x's dtype); Tyr/GPU/Kernels/Rotary.lean:13-66.
+ *   oracle_layernorm_residual  Tyr/GPU/Kernels/FusedLayerNorm.lean:28-140 (out_resid =
+ *                           bf16(x + residual); row statistics of the rounded sum;
+ *                           normalise, weight, bias; bf16 out), in double.
  *   oracle_e4m3_*           OCP FP8 E4M3 ("e4m3fn": bias 7, max 448, no inf, NaN at
  *                           S.1111.111); dtype tag at Tyr/GPU/Types.lean:21-58.
  *
@@ -373,6 +379,65 @@ void oracle_gemm_fp8(const uint8_t* aq, const uint8_t* bq, uint16_t* c, float* c
             if (c_f32) c_f32[m * N + n] = r;
         }
         free(row);
+    }
+}
+
+/* ------------------------------------------------------- rotary / layernorm -- */
+
+/* x, y: [B,S,H,D] as f32 (is_bf16 = 0) or bf16 bit patterns (is_bf16 = 1); cos, sin f32 [S, D/2].
+ * Products and sums are single f32 operations in the order of the reference expression. */
+void oracle_rope(const void* x, const float* cosp, const float* sinp, void* y,
+                 int64_t B, int64_t S, int64_t H, int64_t D, int is_bf16) {
+    const int64_t h = D / 2;
+    for (int64_t row = 0; row < B * S * H; ++row) {
+        const int64_t s = (row / H) % S;
+        for (int64_t i = 0; i < h; ++i) {
+            float x1, x2;
+            if (is_bf16) {
+                x1 = bf16_to_f32(((const uint16_t*)x)[row * D + i]);
+                x2 = bf16_to_f32(((const uint16_t*)x)[row * D + h + i]);
+            } else {
+                x1 = ((const float*)x)[row * D + i];
+                x2 = ((const float*)x)[row * D + h + i];
+            }
+            const float c = cosp[s * h + i], sn = sinp[s * h + i];
+            volatile float a = x1 * c, b = x2 * sn, d = x1 * sn, e = x2 * c;   /* no fused multiply-add */
+            const float y1 = a - b, y2 = d + e;
+            if (is_bf16) {
+                ((uint16_t*)y)[row * D + i] = f32_to_bf16(y1);
+                ((uint16_t*)y)[row * D + h + i] = f32_to_bf16(y2);
+            } else {
+                ((float*)y)[row * D + i] = y1;
+                ((float*)y)[row * D + h + i] = y2;
+            }
+        }
+    }
+}
+
+/* x, residual, out, out_resid: bf16 bit patterns [rows, d]; weight, bias: bf16 [d]. */
+void oracle_layernorm_residual(const uint16_t* x, const uint16_t* residual, const uint16_t* weight,
+                               const uint16_t* bias, uint16_t* out, uint16_t* out_resid,
+                               int64_t rows, int64_t d, double eps) {
+    #pragma omp parallel for
+    for (int64_t r = 0; r < rows; ++r) {
+        double sum = 0.0;
+        for (int64_t i = 0; i < d; ++i) {
+            const uint16_t v = f32_to_bf16(bf16_to_f32(x[r * d + i]) + bf16_to_f32(residual[r * d + i]));
+            out_resid[r * d + i] = v;
+            sum += (double)bf16_to_f32(v);
+        }
+        const double mean = sum / (double)d;
+        double sq = 0.0;
+        for (int64_t i = 0; i < d; ++i) {
+            const double c = (double)bf16_to_f32(out_resid[r * d + i]) - mean;
+            sq += c * c;
+        }
+        const double inv = 1.0 / sqrt(sq / (double)d + eps);
+        for (int64_t i = 0; i < d; ++i) {
+            const double v = ((double)bf16_to_f32(out_resid[r * d + i]) - mean) * inv *
+                             (double)bf16_to_f32(weight[i]) + (double)bf16_to_f32(bias[i]);
+            out[r * d + i] = f32_to_bf16((float)v);
+        }
     }
 }
 

@@ -14,6 +14,7 @@ SYMBOLS = (
     "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
     "tyr_hip_gqa_decode", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
+    "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy",
 )
 
 _lib = None
@@ -55,5 +56,13 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_gemm_bf16.restype = ci
     L.tyr_hip_gemm_fp8.argtypes = [vp, vp, vp, u64, u64, u64, f32, f32, ci, vp]
     L.tyr_hip_gemm_fp8.restype = ci
+    L.tyr_hip_decode_rope_append.argtypes = [vp] * 8 + [u64] * 6 + [vp]
+    L.tyr_hip_decode_rope_append.restype = ci
+    L.tyr_hip_rope_fwd.argtypes = [vp, vp, vp, vp, u64, u64, u64, u64, ci, vp]
+    L.tyr_hip_rope_fwd.restype = ci
+    L.tyr_hip_layernorm_residual.argtypes = [vp] * 6 + [u64, u64, f32, vp]
+    L.tyr_hip_layernorm_residual.restype = ci
+    L.tyr_hip_copy.argtypes = [vp, vp, sz, vp]
+    L.tyr_hip_copy.restype = ci
     _lib = L
     return L

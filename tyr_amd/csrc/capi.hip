@@ -164,6 +164,63 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }
 
+int tyr_hip_decode_rope_append(const void* q, const void* k_new, const void* v_new, const float* cos,
+                               const float* sin, void* q_out, void* k_cache, void* v_cache, uint64_t B,
+                               uint64_t Hq, uint64_t Hkv, uint64_t D, uint64_t kv_stride, uint64_t pos,
+                               void* stream) {
+    if (!q || !k_new || !v_new || !cos || !sin || !q_out || !k_cache || !v_cache) return TYR_HIP_ERR_NULL_POINTER;
+    if (B == 0 || Hq == 0 || Hkv == 0 || D == 0 || pos >= kv_stride) return TYR_HIP_ERR_BAD_SHAPE;
+    if (D % 16 != 0) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!fits_int(D) || !fits_int(B * Hq) || !fits_int(B * Hkv) || !fits_int((B * Hq + 2 * B * Hkv) * (D / 16)))
+        return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(q) || !aligned16(k_new) || !aligned16(v_new) || !aligned16(cos) || !aligned16(sin) ||
+        !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache))
+        return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_decode_rope_append(q, k_new, v_new, cos, sin, q_out, k_cache, v_cache, (int)B,
+                                                  (int)Hq, (int)Hkv, (int)D, (size_t)kv_stride, (size_t)pos,
+                                                  static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_rope_fwd(const void* x, const float* cos, const float* sin, void* y, uint64_t B, uint64_t S,
+                     uint64_t H, uint64_t D, int dtype, void* stream) {
+    if (!x || !cos || !sin || !y) return TYR_HIP_ERR_NULL_POINTER;
+    if (B == 0 || S == 0 || H == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (dtype != TYR_HIP_F32 && dtype != TYR_HIP_BF16) return TYR_HIP_ERR_UNSUPPORTED;
+    if (D % (dtype == TYR_HIP_BF16 ? 16 : 8) != 0) return TYR_HIP_ERR_UNSUPPORTED;
+    if (!fits_int(S) || !fits_int(H) || !fits_int(D)) return TYR_HIP_ERR_BAD_SHAPE;
+    const uint64_t rows = B * S * H;
+    if (rows / S / H != B || rows * (D / 8) / rows != D / 8 || rows * (D / 8) / 256 > (uint64_t)INT_MAX)
+        return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(cos) || !aligned16(sin) || !aligned16(y)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_rope_fwd(x, cos, sin, y, (size_t)rows, (int)S, (int)H, (int)D,
+                                        dtype == TYR_HIP_BF16, static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_layernorm_residual(const void* x, const void* residual, const void* weight, const void* bias,
+                               void* out, void* out_resid, uint64_t rows, uint64_t d_model, float eps,
+                               void* stream) {
+    if (!x || !residual || !weight || !bias || !out || !out_resid) return TYR_HIP_ERR_NULL_POINTER;
+    if (rows == 0 || d_model == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (d_model % 8 != 0 || d_model > 8192 || !(eps >= 0.0f)) return TYR_HIP_ERR_UNSUPPORTED;
+    if ((rows + 3) / 4 > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(residual) || !aligned16(weight) || !aligned16(bias) || !aligned16(out) ||
+        !aligned16(out_resid))
+        return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_layernorm_residual(x, residual, weight, bias, out, out_resid, (size_t)rows,
+                                                  (int)d_model, eps, static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_copy(const void* src, void* dst, size_t bytes, void* stream) {
+    if (!src || !dst) return TYR_HIP_ERR_NULL_POINTER;
+    if (bytes == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (!aligned16(src) || !aligned16(dst)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
+    return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
 int tyr_hip_gemm_bf16(const void* a, const void* b, void* c, uint64_t M, uint64_t N, uint64_t K,
                       int trans_b, void* stream) {
     if (!a || !b || !c) return TYR_HIP_ERR_NULL_POINTER;

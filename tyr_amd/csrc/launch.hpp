@@ -21,4 +21,13 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
                       int Hq, int Hkv, int L, int D, int64_t kv_stride, float scale, int num_splits,
                       void* workspace, hipStream_t stream);
 
+int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+int launch_rope_fwd(const void* x, const float* cosp, const float* sinp, void* y, size_t rows, int S, int H, int D,
+                    int is_bf16, hipStream_t stream);
+int launch_decode_rope_append(const void* q, const void* k_new, const void* v_new, const float* cosp,
+                              const float* sinp, void* q_out, void* k_cache, void* v_cache, int B, int Hq, int Hkv,
+                              int D, size_t kv_stride, size_t pos, hipStream_t stream);
+int launch_layernorm_residual(const void* x, const void* residual, const void* weight, const void* bias, void* out,
+                              void* out_resid, size_t rows, int d_model, float eps, hipStream_t stream);
+
 }  // namespace tyr

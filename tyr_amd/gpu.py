@@ -142,6 +142,78 @@ def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len:
     return o, lse
 
 
+def decode_rope_append(q, k_new, v_new, cos, sin, k_cache, v_cache, pos: int, stream=None):
+    """qRot = decodeRopeAppend q kNew vNew cos sin kCache vCache pos.
+
+    q bf16 [B,Hq,1,D] (or [B,1,Hq,D]); k_new, v_new bf16 [B,Hkv,1,D]; cos, sin f32 [1,D/2] (or [D/2]) for
+    position ``pos``; caches bf16 [B,Hkv,maxLen,D], row ``pos`` of each is overwritten in place.  Returns the
+    rotated q with q's shape."""
+    for t, n in ((q, "q"), (k_new, "kNew"), (v_new, "vNew"), (k_cache, "kCache"), (v_cache, "vCache")):
+        _check(t, n, torch.bfloat16, 4)
+    _check(cos, "cos", torch.float32)
+    _check(sin, "sin", torch.float32)
+    B, Hkv, Lmax, D = k_cache.shape
+    if v_cache.shape != k_cache.shape:
+        raise TyrGpuError("k and v caches must have the same shape")
+    if q.shape[0] != B or q.shape[-1] != D or q.shape[1] * q.shape[2] * B * D != q.numel() or 1 not in q.shape[1:3]:
+        raise TyrGpuError("q must be [B, Hq, 1, D] or [B, 1, Hq, D]")
+    Hq = q.shape[1] * q.shape[2]
+    for t in (k_new, v_new):
+        if t.numel() != B * Hkv * D or t.shape[-1] != D:
+            raise TyrGpuError("kNew and vNew must hold B*Hkv rows of D elements")
+    if cos.numel() != D // 2 or sin.numel() != D // 2:
+        raise TyrGpuError("cos and sin must hold D/2 elements (the table row of this position)")
+    if not 0 <= pos < Lmax:
+        raise TyrGpuError("pos is outside the cache")
+    q_out = torch.empty_like(q)
+    rc = _lib.load().tyr_hip_decode_rope_append(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), cos.data_ptr(),
+                                                sin.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(),
+                                                v_cache.data_ptr(), B, Hq, Hkv, D, Lmax, int(pos), _stream(stream))
+    _raise(rc, "decodeRopeAppend")
+    return q_out
+
+
+def rope_fwd(x, cos, sin, stream=None):
+    """y = applyRotaryEmb x cos sin.  x f32 or bf16 [B,S,H,D]; cos, sin f32 [S,D/2]."""
+    if x.dtype not in (torch.float32, torch.bfloat16):
+        raise TyrGpuError("x must have dtype float32 or bfloat16")
+    _check(x, "x", x.dtype, 4)
+    _check(cos, "cos", torch.float32, 2)
+    _check(sin, "sin", torch.float32, 2)
+    B, S, H, D = x.shape
+    if tuple(cos.shape) != (S, D // 2) or tuple(sin.shape) != (S, D // 2):
+        raise TyrGpuError("cos and sin must have shape [S, D/2]")
+    y = torch.empty_like(x)
+    rc = _lib.load().tyr_hip_rope_fwd(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), y.data_ptr(), B, S, H, D,
+                                      1 if x.dtype == torch.bfloat16 else 0, _stream(stream))
+    _raise(rc, "applyRotaryEmb")
+    return y
+
+
+def layernorm_residual(x, residual, weight, bias, eps: float = 1e-5, stream=None):
+    """(out, outResid) = fusedLayerNormResidual x residual weight bias.  bf16; x, residual [..., d]; weight, bias [d]."""
+    for t, n in ((x, "x"), (residual, "residual"), (weight, "weight"), (bias, "bias")):
+        _check(t, n, torch.bfloat16)
+    d = x.shape[-1]
+    if residual.shape != x.shape or tuple(weight.shape) != (d,) or tuple(bias.shape) != (d,):
+        raise TyrGpuError("residual must match x, weight and bias must be [d_model]")
+    out, out_resid = torch.empty_like(x), torch.empty_like(x)
+    rc = _lib.load().tyr_hip_layernorm_residual(x.data_ptr(), residual.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                                out.data_ptr(), out_resid.data_ptr(), x.numel() // d, d, float(eps),
+                                                _stream(stream))
+    _raise(rc, "fusedLayerNormResidual")
+    return out, out_resid
+
+
+def copy(src, stream=None):
+    """out = copy src (any dtype, contiguous)."""
+    _check(src, "input", src.dtype)
+    dst = torch.empty_like(src)
+    rc = _lib.load().tyr_hip_copy(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(), _stream(stream))
+    _raise(rc, "copy")
+    return dst
+
+
 def gemm_bf16(a, b, trans_b: bool = False, stream=None):
     """C = gemmBf16 a b.  a bf16 [M,K]; b bf16 [K,N] (or [N,K] with trans_b) -> bf16 [M,N]."""
     _check(a, "a", torch.bfloat16, 2)
