@@ -87,12 +87,12 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
             const int row = min(row0 + 16 * T + x, L - 1);
             const uint16_t* kp = Kb + (size_t)row * D + g * 8;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) bf.k[T][i] = ld_global_16(kp + i * 32);
+            for (int i = 0; i < 4; ++i) bf.k[T][i] = ld_global_16_nt(kp + i * 32);
         }
 #pragma unroll
         for (int p = 0; p < 8; ++p) {
             const int row = min(row0 + 16 * (p >> 2) + 4 * g + (p & 3), L - 1);
-            bf.v[p] = ld_global_16(Vb + (size_t)row * D + x * 8);
+            bf.v[p] = ld_global_16_nt(Vb + (size_t)row * D + x * 8);
         }
     };
 

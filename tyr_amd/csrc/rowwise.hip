@@ -87,12 +87,12 @@ __global__ __launch_bounds__(rw::THREADS) void copy_kernel(const u32x4* __restri
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
-            if (i < n16) v[k] = __builtin_nontemporal_load(src + i);
+            if (i < n16) v[k] = ld_global_16_nt(src + i);
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
-            if (i < n16) __builtin_nontemporal_store(v[k], dst + i);
+            if (i < n16) st_global_16_nt(dst + i, v[k]);
         }
     }
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
@@ -112,11 +112,11 @@ __global__ __launch_bounds__(rw::THREADS) void rope_kernel(const T* __restrict__
     const int e0 = (int)(id % per_row) * E;
     const int s = (int)((row / H) % S);
     const T* xr = x + row * D;
-    u32x4 a = ld_global_16(xr + e0), b = ld_global_16(xr + D / 2 + e0);
+    u32x4 a = ld_global_16_nt(xr + e0), b = ld_global_16_nt(xr + D / 2 + e0);
     rw::Piece<T>::rotate(a, b, cosp + (size_t)s * (D / 2) + e0, sinp + (size_t)s * (D / 2) + e0);
     T* yr = y + row * D;
-    st_global_16(yr + e0, a);
-    st_global_16(yr + D / 2 + e0, b);
+    st_global_16_nt(yr + e0, a);
+    st_global_16_nt(yr + D / 2 + e0, b);
 }
 
 // Rows 0 .. B*Hq-1: q rows (rotated into q_out).  Then B*Hkv k rows (rotated into row `pos` of the
@@ -170,12 +170,12 @@ __global__ __launch_bounds__(rw::THREADS) void layernorm_residual_kernel(
         const int pc = lane + 64 * p;
         if (pc < pieces) {
             float a[8], b[8];
-            rw::unpack8(ld_global_16(xr + pc * 8), a);
-            rw::unpack8(ld_global_16(rr + pc * 8), b);
+            rw::unpack8(ld_global_16_nt(xr + pc * 8), a);
+            rw::unpack8(ld_global_16_nt(rr + pc * 8), b);
 #pragma unroll
             for (int i = 0; i < 8; ++i) a[i] += b[i];
             const u32x4 r16 = rw::pack8(a);                     // out_resid is the bf16-rounded sum ...
-            st_global_16(out_resid + row * d_model + pc * 8, r16);
+            st_global_16_nt(out_resid + row * d_model + pc * 8, r16);
             rw::unpack8(r16, v[p]);                             // ... and the statistics are taken from it
 #pragma unroll
             for (int i = 0; i < 8; ++i) sum += v[p][i];
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(rw::THREADS) void layernorm_residual_kernel(
             rw::unpack8(ld_global_16(bias + pc * 8), b);
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = (v[p][i] - mean) * inv_std * w[i] + b[i];
-            st_global_16(out + row * d_model + pc * 8, rw::pack8(o));
+            st_global_16_nt(out + row * d_model + pc * 8, rw::pack8(o));
         }
     }
 }
