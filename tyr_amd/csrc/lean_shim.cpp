@@ -149,6 +149,89 @@ lean_object* lean_tyr_gpu_gqa_decode(uint64_t B, uint64_t Hq, uint64_t Hkv, uint
     }
 }
 
+// decodeRopeAppend {B Hq Hkv L D} q kNew vNew cos sin kCache vCache pos stream : IO (T #[B,Hq,1,D])
+// The caches are mutated in place (row `pos`), like the output tensors of the reference's launchers.
+lean_object* lean_tyr_gpu_decode_rope_append(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                                             b_lean_obj_arg q, b_lean_obj_arg k_new, b_lean_obj_arg v_new,
+                                             b_lean_obj_arg cos, b_lean_obj_arg sin, b_lean_obj_arg k_cache,
+                                             b_lean_obj_arg v_cache, uint64_t pos, uint64_t stream,
+                                             lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), kn = borrowTensor(k_new), vn = borrowTensor(v_new);
+        auto c_ = borrowTensor(cos), s_ = borrowTensor(sin), kc = borrowTensor(k_cache), vc = borrowTensor(v_cache);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(kn, "kNew", torch::kBFloat16, err) ||
+            !check(vn, "vNew", torch::kBFloat16, err) || !check(c_, "cos", torch::kFloat32, err) ||
+            !check(s_, "sin", torch::kFloat32, err) || !check(kc, "kCache", torch::kBFloat16, err) ||
+            !check(vc, "vCache", torch::kBFloat16, err))
+            return io_error(err);
+        auto q_out = torch::empty_like(q_);
+        const int rc = tyr_hip_decode_rope_append(q_.data_ptr(), kn.data_ptr(), vn.data_ptr(), c_.data_ptr<float>(),
+                                                  s_.data_ptr<float>(), q_out.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                  B, Hq, Hkv, D, L, pos, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("decodeRopeAppend", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(q_out)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// applyRotaryEmb {B S H D} x cos sin stream : IO (T #[B,S,H,D])
+lean_object* lean_tyr_gpu_rope_fwd(uint64_t B, uint64_t S, uint64_t H, uint64_t D, b_lean_obj_arg x,
+                                   b_lean_obj_arg cos, b_lean_obj_arg sin, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto x_ = borrowTensor(x), c_ = borrowTensor(cos), s_ = borrowTensor(sin);
+        std::string err;
+        const bool bf16 = x_.scalar_type() == torch::kBFloat16;
+        if (!check(x_, "x", bf16 ? torch::kBFloat16 : torch::kFloat32, err) ||
+            !check(c_, "cos", torch::kFloat32, err) || !check(s_, "sin", torch::kFloat32, err))
+            return io_error(err);
+        auto y = torch::empty_like(x_);
+        const int rc = tyr_hip_rope_fwd(x_.data_ptr(), c_.data_ptr<float>(), s_.data_ptr<float>(), y.data_ptr(), B, S,
+                                        H, D, bf16 ? TYR_HIP_BF16 : TYR_HIP_F32, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("applyRotaryEmb", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(y)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// fusedLayerNormResidual {rows d} x residual weight bias eps stream : IO (out x outResid)
+lean_object* lean_tyr_gpu_layernorm_residual(uint64_t rows, uint64_t d, b_lean_obj_arg x, b_lean_obj_arg residual,
+                                             b_lean_obj_arg weight, b_lean_obj_arg bias, double eps, uint64_t stream,
+                                             lean_object* /*world*/) {
+    try {
+        auto x_ = borrowTensor(x), r_ = borrowTensor(residual), w_ = borrowTensor(weight), b_ = borrowTensor(bias);
+        std::string err;
+        if (!check(x_, "x", torch::kBFloat16, err) || !check(r_, "residual", torch::kBFloat16, err) ||
+            !check(w_, "weight", torch::kBFloat16, err) || !check(b_, "bias", torch::kBFloat16, err))
+            return io_error(err);
+        auto out = torch::empty_like(x_), out_resid = torch::empty_like(x_);
+        const int rc = tyr_hip_layernorm_residual(x_.data_ptr(), r_.data_ptr(), w_.data_ptr(), b_.data_ptr(),
+                                                  out.data_ptr(), out_resid.data_ptr(), rows, d, (float)eps,
+                                                  reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("fusedLayerNormResidual", rc);
+        return pair_result(std::move(out), std::move(out_resid));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// copy {s} input stream : IO (T s)      (the erased shape argument arrives as an owned object and is ignored)
+lean_object* lean_tyr_gpu_copy(lean_obj_arg /*shape*/, b_lean_obj_arg input, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto in_ = borrowTensor(input);
+        if (!in_.is_cuda()) return io_error("input must be a CUDA tensor");
+        if (!in_.is_contiguous()) return io_error("input must be contiguous");
+        auto out = torch::empty_like(in_);
+        const int rc = tyr_hip_copy(in_.data_ptr(), out.data_ptr(), (size_t)in_.nbytes(), reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("copy", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(out)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 // gemmBf16 {M N K} a b stream : IO (T #[M,N])
 lean_object* lean_tyr_gpu_gemm_bf16(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a,
                                     b_lean_obj_arg b, uint64_t stream, lean_object* /*world*/) {

@@ -63,6 +63,34 @@ opaque flashAttnBwd {B H N D : UInt64} (q k v o : @& T #[B, H, N, D]) (lse : @& 
 opaque gqaDecode {B Hq Hkv L D : UInt64} (q : @& T #[B, Hq, 1, D]) (k v : @& T #[B, Hkv, L, D])
     (scale : Float) (numSplits : UInt64) (stream : CudaStream) : IO (T #[B, Hq, 1, D] × T #[B, Hq])
 
+/-- Decode step between the projections and `gqaDecode`: rotary embedding of the single-token `q` and
+    `kNew` (`cos sin : f32 [1, D/2]`, the table row of position `pos`), then `kNew` (rotated) and `vNew`
+    are written into row `pos` of the preallocated caches **in place**. Returns the rotated `q`.
+    Fuses `rotary.applyRotaryEmb` ×2 and `data.sliceScatter` ×2 of `QwenAttention.forwardStep`
+    (`Tyr/Model/Qwen/Attention.lean:172-196`); follow with `gqaDecode` over the first `pos+1` rows. -/
+@[extern "lean_tyr_gpu_decode_rope_append"]
+opaque decodeRopeAppend {B Hq Hkv L D : UInt64} (q : @& T #[B, Hq, 1, D]) (kNew vNew : @& T #[B, Hkv, 1, D])
+    (cos sin : @& T #[1, D / 2]) (kCache vCache : @& T #[B, Hkv, L, D]) (pos : UInt64) (stream : CudaStream)
+    : IO (T #[B, Hq, 1, D])
+
+/-- Rotary embedding, `x : f32 | bf16 [B,S,H,D]`, `cos sin : f32 [S, D/2]`; GPU twin of
+    `rotary.applyRotaryEmb` (`Tyr/Torch.lean:1044`, `cc/src/tyr.cpp:3837-3873`) and of the DSL kernel
+    `rotaryFwd` (`Tyr/GPU/Kernels/Rotary.lean:13-66`). -/
+@[extern "lean_tyr_gpu_rope_fwd"]
+opaque applyRotaryEmb {B S H D : UInt64} (x : @& T #[B, S, H, D]) (cos sin : @& T #[S, D / 2])
+    (stream : CudaStream) : IO (T #[B, S, H, D])
+
+/-- Fused residual add + LayerNorm over the last axis, bf16: returns `(out, outResid)` with
+    `outResid = x + residual`. Replaces `tkFusedLayerNormResidual1024`
+    (`Tyr/GPU/Kernels/FusedLayerNorm.lean:28-140`) for any `rows` and `d ≤ 8192`, `d % 8 = 0`. -/
+@[extern "lean_tyr_gpu_layernorm_residual"]
+opaque fusedLayerNormResidual {rows d : UInt64} (x residual : @& T #[rows, d]) (weight bias : @& T #[d])
+    (eps : Float) (stream : CudaStream) : IO (T #[rows, d] × T #[rows, d])
+
+/-- Device copy; replaces `copy64x64` (`Tyr/GPU/Kernels/Copy.lean:16-27`) for any contiguous tensor. -/
+@[extern "lean_tyr_gpu_copy"]
+opaque copy {s : Shape} (input : @& T s) (stream : CudaStream) : IO (T s)
+
 /-- `C = A · B`, bf16 operands, f32 accumulation, bf16 result; `b` is `K × N` row-major.
     GPU twin of `nn.mm` (`Tyr/Torch.lean:546`). -/
 @[extern "lean_tyr_gpu_gemm_bf16"]
