@@ -131,6 +131,25 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
                        uint64_t kv_stride, float scale, uint64_t num_splits,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* GQA decode with a per-sequence cache length and / or a sliding window.
+ *
+ * Decode-time (one query token) form of `lean_torch_sdpa_gqa_mask` (padding mask: the valid
+ * keys of sequence b are a prefix of the cache; cc/src/tyr.cpp:4019-4095) and of
+ * `lean_torch_sdpa_gqa_window` (position i attends to j <= i with i - j < window;
+ * cc/src/tyr.cpp:3953-4016), the query standing at the last valid position:
+ * sequence b attends to cache rows [max(0, len_b - window), len_b), len_b = kv_lens[b].
+ *
+ *   kv_lens : device int32 [B], each clamped to [1, L]; NULL = every sequence has L rows
+ *   window  : 0 = unbounded
+ *   L       : upper bound of the lengths (sizes the splits and the workspace)
+ * Everything else as tyr_hip_gqa_decode, which is this call with kv_lens = NULL, window = 0.
+ */
+int tyr_hip_gqa_decode_varlen(const void* q, const void* k, const void* v, void* o, float* lse,
+                              uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                              uint64_t kv_stride, const int32_t* kv_lens, uint64_t window,
+                              float scale, uint64_t num_splits, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Decode step: rotary embedding of the new q and k, append of k and v to the cache.
  *

@@ -194,6 +194,35 @@ def test_gqa_decode_equals_last_row_of_causal_prefill(gpu):
     assert max_abs(lse_dec, lse_pre[:, :, -1]) <= 1e-3
 
 
+@pytest.mark.parametrize("window", [0, 1, 37, 256, 5000])
+@pytest.mark.parametrize("splits", [0, 1, 5])
+def test_gqa_decode_varlen_and_window(gpu, window, splits):
+    # Per-sequence cache lengths (the decode-time form of the reference's padding-mask SDPA,
+    # cc/src/tyr.cpp:4019-4095) and a sliding window (cc/src/tyr.cpp:3953-4016): sequence b attends to
+    # rows [max(0, len_b - window), len_b).  Checked by slicing exactly those rows out on the host and
+    # running the checker (and the LibTorch sequence) on the slice.
+    B, Hq, Hkv, Lmax, D = 5, 8, 2, 700, 128
+    lens = [700, 1, 333, 64, 513]
+    q, = lt.make_inputs(900 + window, (B, Hq, 1, D))
+    k, v = lt.make_inputs(901 + window, (B, Hkv, Lmax, D), (B, Hkv, Lmax, D))
+    sc = 1 / math.sqrt(D)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    o, lse = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits, kv_lens=lens_d, window=window)
+    for b, n in enumerate(lens):
+        lo = max(0, n - window) if window > 0 else 0
+        kb, vb = k[b:b + 1, :, lo:n].contiguous(), v[b:b + 1, :, lo:n].contiguous()
+        wo, wl = oracle.gqa_decode(bits(q[b:b + 1]), bits(kb), bits(vb), sc, 1)
+        assert max_abs(o[b:b + 1].cpu().float(), from_bits(wo).float()) <= TOL, (b, n, lo)
+        assert max_abs(lse[b:b + 1].cpu(), wl) <= 1e-3, (b, n, lo)
+        ref = lt.sdpa_gqa_qkv(q[b:b + 1].float(), kb.float(), vb.float(), False, True)
+        assert max_abs(o[b:b + 1].cpu().float(), ref) <= TOL
+    # kv_lens = None with window = 0 is the plain call
+    o0, _ = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits)
+    full = torch.full((B,), Lmax, dtype=torch.int32, device="cuda")
+    o1, _ = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits, kv_lens=full)
+    assert torch.equal(o0, o1)
+
+
 def test_gqa_decode_full_size_config(gpu):
     # batch 32, 32 query heads, 8 kv heads, D=128, contiguous cache of 8192 per sequence.
     B, Hq, Hkv, L, D = 32, 32, 8, 8192, 128

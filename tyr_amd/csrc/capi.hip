@@ -146,6 +146,14 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
                        uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
                        uint64_t kv_stride, float scale, uint64_t num_splits, void* workspace,
                        size_t workspace_bytes, void* stream) {
+    return tyr_hip_gqa_decode_varlen(q, k, v, o, lse, B, Hq, Hkv, L, D, kv_stride, nullptr, 0, scale,
+                                     num_splits, workspace, workspace_bytes, stream);
+}
+
+int tyr_hip_gqa_decode_varlen(const void* q, const void* k, const void* v, void* o, float* lse,
+                              uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                              uint64_t kv_stride, const int32_t* kv_lens, uint64_t window, float scale,
+                              uint64_t num_splits, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
     if (B == 0 || Hq == 0 || Hkv == 0 || L == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (Hq % Hkv != 0 || kv_stride < L) return TYR_HIP_ERR_BAD_SHAPE;
@@ -154,12 +162,14 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
     if (!fits_int(L) || !fits_int(B * Hq) || B * Hkv > 65535 || kv_stride > (uint64_t)INT_MAX)
         return TYR_HIP_ERR_BAD_SHAPE;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
-    if (num_splits == 0) num_splits = auto_splits(B, Hkv, L);
+    if (kv_lens && (reinterpret_cast<uintptr_t>(kv_lens) & 3u)) return TYR_HIP_ERR_MISALIGNED;
+    if (num_splits == 0) num_splits = auto_splits(B, Hkv, window > 0 && window < L ? window : L);
     const size_t need = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
     if (!workspace || workspace_bytes < need) return TYR_HIP_ERR_WORKSPACE;
     if (!aligned16(workspace)) return TYR_HIP_ERR_MISALIGNED;
     const int rc = tyr::launch_gqa_decode(q, k, v, o, lse, (int)B, (int)Hq, (int)Hkv, (int)L, (int)D,
-                                          (int64_t)kv_stride, scale, (int)num_splits, workspace,
+                                          (int64_t)kv_stride, scale, (int)num_splits, workspace, kv_lens,
+                                          (int)(window > (uint64_t)INT_MAX ? INT_MAX : window),
                                           static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }

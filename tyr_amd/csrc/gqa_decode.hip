@@ -43,7 +43,8 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     float* __restrict__ part_o, float* __restrict__ part_m, float* __restrict__ part_l,
     uint16_t* __restrict__ O, float* __restrict__ LSE,
-    int Hq, int Hkv, int G, int L, long kv_stride, int S, int chunk, int wchunk, float scale_log2) {
+    int Hq, int Hkv, int G, int L, long kv_stride, int S, int chunk, int wchunk, float scale_log2,
+    const int* __restrict__ kv_lens, int window) {
     using namespace dec;
     constexpr int THREADS = 64 * WAVES;
     extern __shared__ __attribute__((aligned(16))) float smem[];   // [WAVES][G][D] O, then [WAVES][QPAD] m, l
@@ -58,7 +59,11 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const uint16_t* Kb = Kp + (size_t)bg * kv_stride * D;
     const uint16_t* Vb = Vp + (size_t)bg * kv_stride * D;
 
-    const int c0 = split * chunk;
+    // Per-sequence length (a padding mask over the cache tail) and sliding window: this sequence
+    // attends to cache rows [lo, L).
+    if (kv_lens != nullptr) L = max(1, min(L, kv_lens[b]));
+    const int lo = window > 0 ? max(0, L - window) : 0;
+    const int c0 = lo + split * chunk;
     const int c1 = min(L, c0 + chunk);
     const int r0 = c0 + w * wchunk;             // this wave's rows [r0, r1)
     const int r1 = min(c1, r0 + wchunk);
@@ -232,13 +237,14 @@ __global__ __launch_bounds__(dec::D) void gqa_decode_combine_kernel(
 
 int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                       int Hq, int Hkv, int L, int D, int64_t kv_stride, float scale, int num_splits,
-                      void* workspace, hipStream_t stream) {
+                      void* workspace, const int* kv_lens, int window, hipStream_t stream) {
     using namespace dec;
     (void)D;
     constexpr int WAVES = 8;
     const int G = Hq / Hkv;
     const int S = num_splits;
-    int chunk = (L + S - 1) / S;
+    const int span = window > 0 ? (window < L ? window : L) : L;     // longest range any sequence reads
+    int chunk = (span + S - 1) / S;
     chunk = (chunk + STEP - 1) / STEP * STEP;
     int wchunk = (chunk + WAVES - 1) / WAVES;
     wchunk = (wchunk + STEP - 1) / STEP * STEP;
@@ -257,7 +263,7 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
                        static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k),
                        static_cast<const uint16_t*>(v), part_o, part_m, part_l,
                        static_cast<uint16_t*>(o), lse, Hq, Hkv, G, L, (long)kv_stride, S, chunk, wchunk,
-                       scale * LOG2E);
+                       scale * LOG2E, kv_lens, window);
     if (hipGetLastError() != hipSuccess) return -1;
     if (S > 1) {
         hipLaunchKernelGGL(gqa_decode_combine_kernel, dim3((unsigned)(B * Hq)), dim3(dec::D), 0, stream,

@@ -19,7 +19,7 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
                           int causal, float scale, void* workspace, hipStream_t stream);
 int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                       int Hq, int Hkv, int L, int D, int64_t kv_stride, float scale, int num_splits,
-                      void* workspace, hipStream_t stream);
+                      void* workspace, const int* kv_lens, int window, hipStream_t stream);
 
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 int launch_rope_fwd(const void* x, const float* cosp, const float* sinp, void* y, size_t rows, int S, int H, int D,

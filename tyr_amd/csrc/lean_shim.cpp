@@ -149,6 +149,32 @@ lean_object* lean_tyr_gpu_gqa_decode(uint64_t B, uint64_t Hq, uint64_t Hkv, uint
     }
 }
 
+// gqaDecodeVarlen {B Hq Hkv L D} q k v kvLens window scale numSplits stream : IO (T #[B,Hq,1,D] x T #[B,Hq])
+lean_object* lean_tyr_gpu_gqa_decode_varlen(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                                            b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                            b_lean_obj_arg kv_lens, uint64_t window, double scale,
+                                            uint64_t num_splits, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v), n_ = borrowTensor(kv_lens);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err) || !check(n_, "kvLens", torch::kInt32, err))
+            return io_error(err);
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)Hq}, q_.options().dtype(torch::kFloat32));
+        const size_t ws_bytes = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
+        auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
+        const int rc = tyr_hip_gqa_decode_varlen(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                                 lse.data_ptr<float>(), B, Hq, Hkv, L, D, /*kv_stride=*/L,
+                                                 n_.data_ptr<int32_t>(), window, (float)scale, num_splits,
+                                                 ws.data_ptr(), ws_bytes, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gqaDecodeVarlen", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 // decodeRopeAppend {B Hq Hkv L D} q kNew vNew cos sin kCache vCache pos stream : IO (T #[B,Hq,1,D])
 // The caches are mutated in place (row `pos`), like the output tensors of the reference's launchers.
 lean_object* lean_tyr_gpu_decode_rope_append(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,

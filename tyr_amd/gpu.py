@@ -113,11 +113,13 @@ def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | Non
 
 
 def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len: int | None = None,
-               stream=None):
+               kv_lens=None, window: int = 0, stream=None):
     """O, LSE = gqaDecode q k v scale numSplits.
 
     q bf16 [B,Hq,1,D]; k, v bf16 [B,Hkv,Lmax,D] (the preallocated cache); the first ``kv_len``
-    rows (default all) of every (batch, kv head) are attended to.  -> (bf16 [B,Hq,1,D], f32 [B,Hq]).
+    rows (default all) of every (batch, kv head) are attended to.  ``kv_lens`` (int32 [B] on the device)
+    gives every sequence its own length <= kv_len; ``window`` > 0 restricts each sequence to its last
+    ``window`` rows.  -> (bf16 [B,Hq,1,D], f32 [B,Hq]).
     """
     for t, n in ((q, "q"), (k, "k"), (v, "v")):
         _check(t, n, torch.bfloat16, 4)
@@ -135,9 +137,15 @@ def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len:
     lse = torch.empty((B, Hq), dtype=torch.float32, device=q.device)
     nbytes = lib.tyr_hip_gqa_decode_workspace_bytes(B, Hq, max(Hkv, 1), max(L, 1), D, int(num_splits))
     ws = torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=q.device)
-    rc = lib.tyr_hip_gqa_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-                                B, Hq, Hkv, L, D, Lmax, float(scale), int(num_splits), ws.data_ptr(),
-                                ws.numel(), _stream(stream))
+    lens_ptr = None
+    if kv_lens is not None:
+        _check(kv_lens, "kvLens", torch.int32, 1)
+        if kv_lens.numel() != B:
+            raise TyrGpuError("kvLens must hold one length per sequence")
+        lens_ptr = kv_lens.data_ptr()
+    rc = lib.tyr_hip_gqa_decode_varlen(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                       B, Hq, Hkv, L, D, Lmax, lens_ptr, int(window), float(scale),
+                                       int(num_splits), ws.data_ptr(), ws.numel(), _stream(stream))
     _raise(rc, "gqaDecode")
     return o, lse
 

@@ -63,6 +63,15 @@ opaque flashAttnBwd {B H N D : UInt64} (q k v o : @& T #[B, H, N, D]) (lse : @& 
 opaque gqaDecode {B Hq Hkv L D : UInt64} (q : @& T #[B, Hq, 1, D]) (k v : @& T #[B, Hkv, L, D])
     (scale : Float) (numSplits : UInt64) (stream : CudaStream) : IO (T #[B, Hq, 1, D] × T #[B, Hq])
 
+/-- `gqaDecode` with a per-sequence cache length (`kvLens : int32 [B]`, a padding mask over the cache
+    tail) and a sliding window (`window = 0`: unbounded): sequence `b` attends to cache rows
+    `[max 0 (kvLens[b] - window), kvLens[b])`. Decode-time form of `nn.scaledDotProductAttentionGQAMask` and
+    `nn.scaledDotProductAttentionGQAWindow` (`cc/src/tyr.cpp:3953-4095`). -/
+@[extern "lean_tyr_gpu_gqa_decode_varlen"]
+opaque gqaDecodeVarlen {B Hq Hkv L D : UInt64} (q : @& T #[B, Hq, 1, D]) (k v : @& T #[B, Hkv, L, D])
+    (kvLens : @& T #[B]) (window : UInt64) (scale : Float) (numSplits : UInt64) (stream : CudaStream)
+    : IO (T #[B, Hq, 1, D] × T #[B, Hq])
+
 /-- Decode step between the projections and `gqaDecode`: rotary embedding of the single-token `q` and
     `kNew` (`cos sin : f32 [1, D/2]`, the table row of position `pos`), then `kNew` (rotated) and `vNew`
     are written into row `pos` of the preallocated caches **in place**. Returns the rotated `q`.
