@@ -75,6 +75,27 @@ int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
                            uint64_t B, uint64_t H, uint64_t N, uint64_t D,
                            int causal, float scale, void* stream);
 
+/* Flash-attention forward with grouped queries, sliding window and per-sequence key length.
+ *
+ * GPU twin of the prefill calls of the reference's models: `lean_torch_sdpa_gqa`
+ * (cc/src/tyr.cpp:3913-3949: K / V repeat_interleave'd along the head axis, query head h
+ * reads kv head h / (Hq/Hkv); caller Tyr/Model/Qwen/Attention.lean:138),
+ * `lean_torch_sdpa_gqa_window` (cc/src/tyr.cpp:3953-4016: key j visible to query i iff
+ * j <= i and i - j < window) and `lean_torch_sdpa_gqa_mask` (cc/src/tyr.cpp:4019-4095)
+ * for padding masks whose valid keys are a prefix of the sequence.
+ *
+ *   q, o   : bf16 [B, Hq, N, D]      k, v : bf16 [B, Hkv, N, D], Hq % Hkv == 0
+ *   window : 0 = none; > 0 requires causal != 0
+ *   kv_lens: device int32 [B] (valid key count of each sequence, clamped to [1, N]) or NULL.
+ *            Keys at or beyond it are masked; rows of padded queries are still written
+ *            (a row that sees no key at all gets O = 0, LSE = -inf).
+ * tyr_hip_flash_attn_fwd is this call with Hkv = Hq, window = 0, kv_lens = NULL.
+ */
+int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void* o, float* lse,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* stream);
+
 /* ---------------------------------------------------------------------------
  * Flash-attention backward.
  *

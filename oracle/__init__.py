@@ -46,6 +46,8 @@ def lib() -> ctypes.CDLL:
                                  ctypes.c_void_p, ctypes.c_int)
         L.oracle_attn_fwd_f64.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
         L.oracle_attn_fwd_f64.restype = None
+        L.oracle_attn_fwd_f64_ex.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, i64, vp, f64]
+        L.oracle_attn_fwd_f64_ex.restype = None
         L.oracle_attn_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
         L.oracle_attn_bwd_f64.restype = None
         L.oracle_attn_fwd_tiled.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f32, i64]
@@ -119,6 +121,20 @@ def attn_fwd_f64(q, k, v, causal: bool, scale: float):
     o = np.empty((B, H, N, D), np.float32)
     lse = np.empty((B, H, N), np.float32)
     lib().oracle_attn_fwd_f64(_p(q), _p(k), _p(v), _p(o), _p(lse), B, H, N, D, int(causal), float(scale))
+    return o, lse
+
+
+def attn_fwd_f64_ex(q, k, v, causal: bool, scale: float, window: int = 0, kv_lens=None):
+    """Double-precision attention with grouped queries (k, v may have fewer heads), a sliding window and
+    per-sequence key lengths (int32 [B]).  -> (O f32 [B,Hq,N,D], LSE f32 [B,Hq,N])."""
+    q, k, v = (_chk(t, np.uint16, n) for t, n in ((q, "q"), (k, "k"), (v, "v")))
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    o = np.empty((B, Hq, N, D), np.float32)
+    lse = np.empty((B, Hq, N), np.float32)
+    lens = None if kv_lens is None else _chk(np.asarray(kv_lens, dtype=np.int32), np.int32, "kv_lens")
+    lib().oracle_attn_fwd_f64_ex(_p(q), _p(k), _p(v), _p(o), _p(lse), B, Hq, Hkv, N, D, int(causal), int(window),
+                                 None if lens is None else _p(lens), float(scale))
     return o, lse
 
 

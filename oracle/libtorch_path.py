@@ -95,6 +95,46 @@ def decode_step_cache_update(q, k_new, v_new, cos, sin, k_cache, v_cache, pos: i
     return q_rot, k2, v2
 
 
+def sdpa_gqa(q, k, v, is_causal: bool, enable_gqa: bool = True, dropout_p: float = 0.0):
+    """The call sequence of lean_torch_sdpa_gqa (equal q and kv lengths)."""
+    return sdpa_gqa_qkv(q, k, v, is_causal, enable_gqa, dropout_p)
+
+
+def _repeat_kv(q, k, v):
+    n_head, n_kv_head = q.shape[1], k.shape[1]
+    if n_head != n_kv_head and n_kv_head > 0:
+        rep = n_head // n_kv_head
+        k, v = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
+    return k, v
+
+
+def sdpa_gqa_window(q, k, v, window_size: int):
+    """The call sequence of lean_torch_sdpa_gqa_window: explicit -inf / 0 mask from
+    (col > row) | (row - col >= window)."""
+    k, v = _repeat_kv(q, k, v)
+    n = q.size(2)
+    row = torch.arange(n).unsqueeze(1)
+    col = torch.arange(n).unsqueeze(0)
+    combined = (col > row) | ((row - col) >= int(window_size))
+    mask = torch.where(combined, torch.full((n, n), float("-inf"), dtype=q.dtype), torch.zeros((n, n), dtype=q.dtype))
+    return F.scaled_dot_product_attention(q, k, v, mask.unsqueeze(0).unsqueeze(0), 0.0, False)
+
+
+def sdpa_gqa_mask(q, k, v, padding_mask, is_causal: bool):
+    """The call sequence of lean_torch_sdpa_gqa_mask: padding_mask [B, N], 1 = valid key."""
+    k, v = _repeat_kv(q, k, v)
+    n = q.size(2)
+    key_mask = padding_mask.unsqueeze(1).unsqueeze(2)
+    if is_causal:
+        row = torch.arange(n).unsqueeze(1)
+        col = torch.arange(n).unsqueeze(0)
+        combined = (col > row).unsqueeze(0).unsqueeze(0) | (key_mask == 0)
+    else:
+        combined = (key_mask == 0)
+    mask = torch.where(combined, torch.tensor(float("-inf"), dtype=q.dtype), torch.tensor(0.0, dtype=q.dtype))
+    return F.scaled_dot_product_attention(q, k, v, mask, 0.0, False)
+
+
 def mm(a, b):
     return torch.mm(a, b)
 

@@ -16,6 +16,9 @@
  *   oracle_attn_fwd_f64     textbook softmax(QK^T*scale + mask) V in double; the
  *                           same math as Examples/GPU/RunFlashAttn.lean:31-48
  *                           (reference values for O and LSE).
+ *   oracle_attn_fwd_f64_ex  the same with the grouped-query head mapping of
+ *                           cc/src/tyr.cpp:3913-3949, the window rule of :3953-4016 and a
+ *                           prefix padding mask (:4019-4095).
  *   oracle_attn_bwd_f64     Tyr/GPU/Kernels/MhaH100.lean:197-344 (backward prep
  *                           d = rowsum(dO o O) and the dQ / dK / dV products:
  *                           P = exp(S*scale - lse), dP = dO V^T, dS = P o (dP - d),
@@ -145,6 +148,54 @@ void oracle_attn_fwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v
                 double acc = 0.0;
                 for (int64_t j = 0; j < jmax; ++j) acc += s[j] * (double)bf16_to_f32(v[(bh * N + j) * D + d]);
                 o[(bh * N + i) * D + d] = (float)(acc / l);
+            }
+            if (lse) lse[bh * N + i] = (float)(log(l) + m);
+            free(s);
+        }
+    }
+}
+
+/* Textbook attention in double precision with grouped queries, a sliding window and a
+ * per-sequence key length: q [B,Hq,N,D]; k, v [B,Hkv,N,D]; query head h reads kv head
+ * h / (Hq/Hkv) (repeat_interleave along the head axis, cc/src/tyr.cpp:3930-3936); key j is
+ * visible to query i iff j < kv_lens[b] (if given), j <= i (if causal) and i - j < window
+ * (if window > 0; cc/src/tyr.cpp:3980-3996).  A row without any visible key gets O = 0,
+ * LSE = -inf. */
+void oracle_attn_fwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                            float* o, float* lse, int64_t B, int64_t Hq, int64_t Hkv, int64_t N,
+                            int64_t D, int causal, int64_t window, const int32_t* kv_lens, double scale) {
+    const int64_t G = Hq / Hkv;
+    #pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t bh = 0; bh < B * Hq; ++bh) {
+        for (int64_t i = 0; i < N; ++i) {
+            const int64_t b = bh / Hq, h = bh % Hq, kvh = b * Hkv + h / G;
+            const uint16_t* qr = q + (bh * N + i) * D;
+            int64_t len = kv_lens ? kv_lens[b] : N;
+            if (len > N) len = N;
+            if (len < 1) len = 1;
+            int64_t jhi = causal ? (i + 1 < len ? i + 1 : len) : len;       /* exclusive */
+            int64_t jlo = window > 0 ? (i - window + 1 > 0 ? i - window + 1 : 0) : 0;
+            float* orow = o + (bh * N + i) * D;
+            if (jlo >= jhi) {
+                for (int64_t d = 0; d < D; ++d) orow[d] = 0.0f;
+                if (lse) lse[bh * N + i] = -INFINITY;
+                continue;
+            }
+            double* s = (double*)malloc(sizeof(double) * (size_t)(jhi - jlo));
+            double m = -INFINITY;
+            for (int64_t j = jlo; j < jhi; ++j) {
+                const uint16_t* kr = k + (kvh * N + j) * D;
+                double acc = 0.0;
+                for (int64_t d = 0; d < D; ++d) acc += (double)bf16_to_f32(qr[d]) * (double)bf16_to_f32(kr[d]);
+                s[j - jlo] = acc * scale;
+                if (s[j - jlo] > m) m = s[j - jlo];
+            }
+            double l = 0.0;
+            for (int64_t j = jlo; j < jhi; ++j) { s[j - jlo] = exp(s[j - jlo] - m); l += s[j - jlo]; }
+            for (int64_t d = 0; d < D; ++d) {
+                double acc = 0.0;
+                for (int64_t j = jlo; j < jhi; ++j) acc += s[j - jlo] * (double)bf16_to_f32(v[(kvh * N + j) * D + d]);
+                orow[d] = (float)(acc / l);
             }
             if (lse) lse[bh * N + i] = (float)(log(l) + m);
             free(s);

@@ -128,6 +128,73 @@ def test_flash_attn_full_size_config(gpu):
     assert torch.equal(gpu.flash_attn_fwd(q, k, v, causal=True, scale=sc)[0], o)   # deterministic
 
 
+# ------------------------------------------- grouped queries, window, key lengths (prefill)
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 4, 1, 200, 128), (2, 8, 2, 333, 64), (8, 2, 1, 129, 128), (1, 32, 8, 512, 128)])
+def test_flash_attn_grouped_queries(gpu, B, Hq, Hkv, N, D, causal):
+    # lean_torch_sdpa_gqa: query head h reads kv head h / (Hq/Hkv).  (8,2,1,...) exercises the XCD-dealt mapping.
+    q, = lt.make_inputs(1200 + N, (B, Hq, N, D))
+    k, v = lt.make_inputs(1201 + N, (B, Hkv, N, D), (B, Hkv, N, D))
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc)
+    wo, wl = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, sc)
+    assert max_abs(o.cpu().float(), wo) <= TOL
+    assert max_abs(lse.cpu(), wl) <= TOL
+    # identical to the plain kernel on materialised repeat_interleave'd K / V
+    G = Hq // Hkv
+    o2, lse2 = gpu.flash_attn_fwd(q.cuda(), k.cuda().repeat_interleave(G, 1).contiguous(),
+                                  v.cuda().repeat_interleave(G, 1).contiguous(), causal=causal, scale=sc)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+@pytest.mark.parametrize("window", [1, 31, 72, 250, 4096])
+@pytest.mark.parametrize("N,D", [(600, 128), (257, 64)])
+def test_flash_attn_sliding_window(gpu, window, N, D):
+    # lean_torch_sdpa_gqa_window: key j visible to query i iff j <= i and i - j < window (72 and 250 are the
+    # reference models' windows).
+    B, Hq, Hkv = 2, 4, 2
+    q, = lt.make_inputs(1300 + window, (B, Hq, N, D))
+    k, v = lt.make_inputs(1301 + window, (B, Hkv, N, D), (B, Hkv, N, D))
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=True, scale=sc, window=window)
+    wo, wl = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), True, sc, window=window)
+    assert max_abs(o.cpu().float(), wo) <= TOL
+    assert max_abs(lse.cpu(), wl) <= TOL
+    if window >= N:                                   # a window wider than the sequence is plain causal attention
+        o2, _ = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=True, scale=sc)
+        assert max_abs(o.float(), o2.float()) <= 1e-6
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_attn_key_lengths(gpu, causal):
+    # prefix padding mask (lean_torch_sdpa_gqa_mask): keys at or beyond a sequence's length are masked,
+    # bit-for-bit independent of what the padded keys / values hold.
+    B, Hq, Hkv, N, D = 4, 4, 2, 300, 128
+    lens = [300, 1, 129, 64]
+    q, = lt.make_inputs(1400, (B, Hq, N, D))
+    k, v = lt.make_inputs(1401, (B, Hkv, N, D), (B, Hkv, N, D))
+    sc = 1 / math.sqrt(D)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc, kv_lens=lens_d)
+    wo, wl = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, sc, kv_lens=lens)
+    assert max_abs(o.cpu().float(), wo) <= TOL
+    assert max_abs(lse.cpu(), wl) <= TOL
+    k2, v2 = k.clone(), v.clone()
+    for b, n in enumerate(lens):
+        k2[b, :, n:] = 50.0
+        v2[b, :, n:] = -50.0
+    o2, lse2 = gpu.flash_attn_fwd(q.cuda(), k2.cuda(), v2.cuda(), causal=causal, scale=sc, kv_lens=lens_d)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+    # window and lengths together
+    o3, lse3 = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=True, scale=sc, kv_lens=lens_d, window=40)
+    wo3, wl3 = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), True, sc, window=40, kv_lens=lens)
+    assert max_abs(o3.cpu().float(), wo3) <= TOL
+    finite = np.isfinite(wl3)
+    assert max_abs(lse3.cpu()[torch.from_numpy(finite)], wl3[finite]) <= TOL
+    assert bool(torch.isinf(lse3.cpu()[torch.from_numpy(~finite)]).all())
+
+
 # ------------------------------------------------------------------------- decode
 
 @pytest.mark.parametrize("B,Hq,Hkv,L,splits", [(1, 4, 1, 32, 1), (2, 8, 2, 300, 0), (1, 32, 8, 513, 3),

@@ -185,3 +185,49 @@ def test_decode_equals_last_row_of_causal_prefill():
     dec, lse_dec = oracle.gqa_decode(bits(q[:, :, -1:].contiguous()), bits(k), bits(v), 0.125, 3)
     assert np.abs(from_bits(dec).float().numpy()[:, :, 0] - from_bits(pre).float().numpy()[:, :, -1]).max() <= 4e-3
     np.testing.assert_allclose(lse_dec, lse_pre[:, :, -1], atol=2e-5)
+
+
+# ------------------------------------------------- grouped queries, window, key lengths
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_f64_ex_grouped_queries_equal_repeat_interleave(causal):
+    B, Hq, Hkv, N, D = 2, 6, 2, 45, 16
+    q, = lt.make_inputs(31, (B, Hq, N, D))
+    k, v = lt.make_inputs(32, (B, Hkv, N, D), (B, Hkv, N, D))
+    o, lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25)
+    kr, vr = k.repeat_interleave(3, 1), v.repeat_interleave(3, 1)
+    o2, lse2 = oracle.attn_fwd_f64(bits(q), bits(kr), bits(vr), causal, 0.25)
+    np.testing.assert_array_equal(o, o2)
+    np.testing.assert_array_equal(lse, lse2)
+    ref = lt.sdpa_gqa(q.double(), k.double(), v.double(), causal)
+    np.testing.assert_allclose(o, ref.numpy(), atol=1e-5)
+
+
+@pytest.mark.parametrize("window", [1, 5, 72, 1000])
+def test_f64_ex_window_matches_libtorch_sequence(window):
+    B, Hq, Hkv, N, D = 1, 4, 2, 90, 16
+    q, = lt.make_inputs(33, (B, Hq, N, D))
+    k, v = lt.make_inputs(34, (B, Hkv, N, D), (B, Hkv, N, D))
+    o, lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), True, 0.25, window=window)
+    ref = lt.sdpa_gqa_window(q.double(), k.double(), v.double(), window)
+    np.testing.assert_allclose(o, ref.numpy(), atol=1e-5)
+    if window == 1:                                   # each query sees only itself: O = V, LSE = score
+        np.testing.assert_allclose(o, v.repeat_interleave(2, 1).float().numpy(), atol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_f64_ex_key_lengths_match_libtorch_padding_mask(causal):
+    B, Hq, Hkv, N, D = 3, 2, 1, 40, 16
+    lens = [40, 7, 1]
+    q, = lt.make_inputs(35, (B, Hq, N, D))
+    k, v = lt.make_inputs(36, (B, Hkv, N, D), (B, Hkv, N, D))
+    o, lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25, kv_lens=lens)
+    pm = (torch.arange(N)[None, :] < torch.tensor(lens)[:, None]).long()
+    ref = lt.sdpa_gqa_mask(q.double(), k.double(), v.double(), pm, causal)
+    np.testing.assert_allclose(o, ref.numpy(), atol=1e-5)
+    # changing keys / values beyond a sequence's length changes nothing
+    k2, v2 = k.clone(), v.clone()
+    k2[1, :, 7:] = 9.0
+    v2[1, :, 7:] = -9.0
+    o2, _ = oracle.attn_fwd_f64_ex(bits(q), bits(k2), bits(v2), causal, 0.25, kv_lens=lens)
+    np.testing.assert_array_equal(o, o2)

@@ -11,7 +11,7 @@ LIB_PATH = os.environ.get("TYR_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libt
 # every symbol include/tyr_hip.h declares
 SYMBOLS = (
     "tyr_hip_strerror", "tyr_hip_version", "tyr_hip_device_info", "tyr_hip_check_device_pointer",
-    "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
+    "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_fwd_gqa", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
     "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
     "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy",
@@ -42,6 +42,8 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_check_device_pointer.restype = ci
     L.tyr_hip_flash_attn_fwd.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, ci, f32, vp]
     L.tyr_hip_flash_attn_fwd.restype = ci
+    L.tyr_hip_flash_attn_fwd_gqa.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, u64, ci, u64, vp, f32, vp]
+    L.tyr_hip_flash_attn_fwd_gqa.restype = ci
     L.tyr_hip_flash_attn_bwd_workspace_bytes.argtypes = [u64] * 4
     L.tyr_hip_flash_attn_bwd_workspace_bytes.restype = sz
     L.tyr_hip_flash_attn_bwd.argtypes = [vp] * 9 + [u64] * 4 + [ci, f32, vp, sz, vp]

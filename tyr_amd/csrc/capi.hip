@@ -88,17 +88,27 @@ int tyr_hip_check_device_pointer(const void* p) {
 int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                            uint64_t B, uint64_t H, uint64_t N, uint64_t D, int causal, float scale,
                            void* stream) {
+    return tyr_hip_flash_attn_fwd_gqa(q, k, v, o, lse, B, H, H, N, D, causal, 0, nullptr, scale, stream);
+}
+
+int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void* o, float* lse,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* stream) {
     if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
-    if (B == 0 || H == 0 || N == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (B == 0 || Hq == 0 || Hkv == 0 || N == 0 || D == 0 || Hq % Hkv != 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return TYR_HIP_ERR_UNSUPPORTED;
+    if (window > 0 && !causal) return TYR_HIP_ERR_UNSUPPORTED;        // the window is a causal one
     if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
-    if (!fits_int(N) || !fits_int(B * H) || B * H > (uint64_t)INT_MAX / ((N + 127) / 128))
+    if (!fits_int(N) || !fits_int(B * Hq) || B * Hq > (uint64_t)INT_MAX / ((N + 127) / 128))
         return TYR_HIP_ERR_BAD_SHAPE;
     if (N * D * 2 >= ((uint64_t)1 << 32)) return TYR_HIP_ERR_UNSUPPORTED;   // one head's K or V must stay below 4 GiB
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
     if (lse && (reinterpret_cast<uintptr_t>(lse) & 3u)) return TYR_HIP_ERR_MISALIGNED;
-    const int rc = tyr::launch_flash_attn_fwd(q, k, v, o, lse, (int)B, (int)H, (int)N, (int)D,
-                                              causal != 0, scale, static_cast<hipStream_t>(stream));
+    if (kv_lens && (reinterpret_cast<uintptr_t>(kv_lens) & 3u)) return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_flash_attn_fwd(q, k, v, o, lse, (int)B, (int)Hq, (int)Hkv, (int)N, (int)D,
+                                              causal != 0, (int)(window > (uint64_t)INT_MAX ? INT_MAX : window),
+                                              kv_lens, scale, static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }
 

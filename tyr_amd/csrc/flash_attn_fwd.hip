@@ -30,6 +30,8 @@
 // kv row).  V^T fragments come from ds_read_b64_tr_b16: within each 16-lane block, lane 4q+p
 // receives element p of the 8-byte pieces addressed by lanes q, q+4, q+8, q+12 -- so four lanes
 // pointing at 4 consecutive d of 4 kv rows hand every lane "its" d for those 4 rows.
+#include <limits.h>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -63,10 +65,13 @@ template <int D> __device__ __forceinline__ int k_swz(int row, int c) { return c
 template <int D> __device__ __forceinline__ int v_swz(int row, int c) { return c ^ (((row & 3) << 2) & (Cfg<D>::KCH - 1)); }
 }  // namespace fa
 
-template <int D, bool CAUSAL>
+// EXT adds the per-sequence key length (padding mask over the tail) and the sliding window; the
+// plain instantiation carries none of their instructions.  G = query heads per kv head.
+template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
-    uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2) {
+    uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2,
+    int Hq, int G, int window, const int* __restrict__ kv_lens) {
     using namespace fa;
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -78,29 +83,42 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // workgroup -> (head, query tile).  Heads are dealt to the 8 XCDs so that all query tiles of a
     // head run on one XCD (shared K/V in its L2); within a head the longest (last) causal tiles
     // are issued first.
-    int bh, qt;
+    // With grouped queries (G > 1) the unit dealt to an XCD is a (batch, kv head) group: its G
+    // query heads times ntq tiles share one K/V; the G heads of a tile are adjacent.
+    int bh, qt, kvbh;
     {
         const int id = blockIdx.x;
+        const int ngroups = BH / G;              // B * Hkv
         int tr;
-        if ((BH & 7) == 0) {
+        if ((ngroups & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
-            bh = (slot / ntq) * 8 + xcd;
-            tr = slot % ntq;
+            const int per_group = G * ntq;
+            kvbh = (slot / per_group) * 8 + xcd;
+            const int within = slot % per_group;
+            tr = within / G;
+            const int hkv = Hq / G;
+            bh = (kvbh / hkv) * Hq + (kvbh % hkv) * G + within % G;
         } else {
             bh = id / ntq;
             tr = id % ntq;
+            kvbh = (bh / Hq) * (Hq / G) + (bh % Hq) / G;
         }
         qt = CAUSAL ? ntq - 1 - tr : tr;
     }
     const int q0 = qt * BM;
     const int qw0 = q0 + w * 32;                 // first query row of this wave
     const size_t head_off = (size_t)bh * N * D;
+    const size_t kv_head_off = (size_t)kvbh * N * D;
     const uint16_t* Qh = Q + head_off;
-    const uint16_t* Kh = Kp + head_off;
-    const uint16_t* Vh = Vp + head_off;
+    const uint16_t* Kh = Kp + kv_head_off;
+    const uint16_t* Vh = Vp + kv_head_off;
 
-    const int kv_end = CAUSAL ? min(N, q0 + BM) : N;
-    const int nkv = (kv_end + BN - 1) / BN;
+    // keys at or beyond Nk are masked; with a window, query i sees keys (i - window, i]
+    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    const int kv_end = CAUSAL ? min(Nk, q0 + BM) : Nk;
+    const int nkv_abs = (kv_end + BN - 1) / BN;
+    const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / BN, nkv_abs - 1) : 0;   // first tile any row sees
+    const int nkv = nkv_abs - jbase;             // tiles are numbered from jbase below
 
     // ---- Q^T fragments: lane holds row qw0+r, columns 16i + 8g + [0,8)
     bf16x8 qf[C::KSTEPS];
@@ -148,7 +166,9 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     for (int i = 0; i < C::DT; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[i][e] = 0.0f;
-    float m2 = -INFINITY;      // running row maximum, in log2 units (score * scale * log2 e)
+    // running row maximum, in log2 units (score * scale * log2 e).  With a window a row's first
+    // tiles can be wholly masked; a finite start keeps (-inf) - m2 from becoming NaN there.
+    float m2 = EXT ? -1.0e30f : -INFINITY;
     float lsum = 0.0f;         // this lane's share of the running row sum
 
     // K fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g.
@@ -169,7 +189,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     }
     const int qpos = qw0 + r;
     // number of kv tiles that intersect this wave's visible region
-    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / BN + 1) : nkv;
+    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / BN + 1 - jbase) : nkv;
 
     constexpr int NG = C::KSTEPS / 2;            // S^T is built in NG groups of (2 k-steps x 2 sub-tiles)
     auto read_k_group = [&](const unsigned char* Kt, int grp, bf16x8 (&dst)[4]) {
@@ -189,9 +209,9 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     };
 
     // ---- prologue: K(0), V(0), K(1) in flight; S(0) computed on its own
-    issue_k(0, 0);
-    issue_v(0, 0);
-    if (nkv > 1) issue_k(1, BN);
+    issue_k(0, jbase * BN);
+    issue_v(0, jbase * BN);
+    if (nkv > 1) issue_k(1, (jbase + 1) * BN);
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
     wait_vmcnt0();
@@ -213,7 +233,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // tile j+1 (into `nxt`).  K runs one tile ahead of V in LDS: at entry K(j+1) and V(j) are
     // resident; K(j+2) and V(j+1) are requested here and awaited at the end.
     auto tile_step = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2], int j) {
-        const int j0 = j * BN;
+        const int j0 = (jbase + j) * BN;
         // The two requests are issued apart (K here, V after the row-max reduction) so the waves of
         // a CU do not all queue on the texture path at once.
         if (j + 2 < nkv) issue_k(j & 1, j0 + 2 * BN);
@@ -225,16 +245,18 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
             // ---- mask (diagonal tiles, ragged tail) -- register e of sub-tile T is kv row
             //      j0 + 32T + 8(e/4) + 4g + e%4
-            const bool need_mask = (CAUSAL && (j0 + BN - 1 > qw0)) || (j0 + BN > N);
+            const bool need_mask = (CAUSAL && (j0 + BN - 1 > qw0)) || (j0 + BN > Nk) ||
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
             if (need_mask) {
-                const int lim = CAUSAL ? min(qpos, N - 1) : N - 1;   // largest visible kv row
+                const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;   // largest visible kv row
+                const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;   // smallest visible kv row
                 const int base = j0 + 4 * g;
 #pragma unroll
                 for (int T = 0; T < 2; ++T)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        if (kv > lim) cur[T][e] = -INFINITY;
+                        if (kv > lim || (EXT && kv < low)) cur[T][e] = -INFINITY;
                     }
             }
 
@@ -326,7 +348,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // scratch (all K/V stages are dead after the last barrier) so that global stores are 16 bytes
     // per lane along rows.
     const float ltot = sum_xor32(lsum);
-    const float inv = 1.0f / ltot;
+    const float inv = (!EXT || ltot > 0.0f) ? 1.0f / ltot : 0.0f;    // EXT: a row that saw no key gives 0
     {
         constexpr int SROW = D * 2 + 16;
         unsigned char* scratch = lds + w * (32 * SROW);
@@ -353,9 +375,11 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 }
 
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
-                          int H, int N, int D, int causal, float scale, hipStream_t stream) {
+                          int Hq, int Hkv, int N, int D, int causal, int window, const int* kv_lens,
+                          float scale, hipStream_t stream) {
     using namespace fa;
-    const int BH = B * H;
+    const int BH = B * Hq;
+    const int G = Hq / Hkv;
     const int ntq = (N + BM - 1) / BM;
     dim3 grid((unsigned)(BH * ntq)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
@@ -363,17 +387,23 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
     auto Kp = static_cast<const uint16_t*>(k);
     auto Vp = static_cast<const uint16_t*>(v);
     auto Op = static_cast<uint16_t*>(o);
-#define TYR_FA_LAUNCH(DD, CC)                                                                    \
+    const bool ext = window > 0 || kv_lens != nullptr;
+#define TYR_FA_LAUNCH(DD, CC, EE)                                                                \
     do {                                                                                         \
         static const hipError_t attr = hipFuncSetAttribute(                                      \
-            reinterpret_cast<const void*>(&flash_attn_fwd_kernel<DD, CC>),                       \
+            reinterpret_cast<const void*>(&flash_attn_fwd_kernel<DD, CC, EE>),                   \
             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DD>::LDS);                           \
         if (attr != hipSuccess) return -1;                                                       \
-        hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC>), grid, block, Cfg<DD>::LDS, stream,   \
-                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2);                         \
+        hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC, EE>), grid, block, Cfg<DD>::LDS, stream, \
+                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens);  \
     } while (0)
-    if (D == 128) { if (causal) TYR_FA_LAUNCH(128, true); else TYR_FA_LAUNCH(128, false); }
-    else          { if (causal) TYR_FA_LAUNCH(64, true);  else TYR_FA_LAUNCH(64, false); }
+#define TYR_FA_PICK(DD)                                                                          \
+    do {                                                                                         \
+        if (ext) { if (causal) TYR_FA_LAUNCH(DD, true, true); else TYR_FA_LAUNCH(DD, false, true); }   \
+        else     { if (causal) TYR_FA_LAUNCH(DD, true, false); else TYR_FA_LAUNCH(DD, false, false); } \
+    } while (0)
+    if (D == 128) TYR_FA_PICK(128); else TYR_FA_PICK(64);
+#undef TYR_FA_PICK
 #undef TYR_FA_LAUNCH
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }

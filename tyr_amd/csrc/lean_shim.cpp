@@ -89,6 +89,29 @@ lean_object* lean_tyr_gpu_flash_attn_fwd(uint64_t B, uint64_t H, uint64_t N, uin
     }
 }
 
+// flashAttnFwdGQA {B Hq Hkv N D} q k v kvLens causal window scale stream : IO (T #[B,Hq,N,D] x T #[B,Hq,N])
+lean_object* lean_tyr_gpu_flash_attn_fwd_gqa(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                             b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                             b_lean_obj_arg kv_lens, uint8_t causal, uint64_t window, double scale,
+                                             uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v), n_ = borrowTensor(kv_lens);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err) || !check(n_, "kvLens", torch::kInt32, err))
+            return io_error(err);
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)Hq, (int64_t)N}, q_.options().dtype(torch::kFloat32));
+        const int rc = tyr_hip_flash_attn_fwd_gqa(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                                  lse.data_ptr<float>(), B, Hq, Hkv, N, D, causal, window,
+                                                  n_.data_ptr<int32_t>(), (float)scale, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnFwdGQA", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 // flashAttnBwd {B H N D} q k v o lse dO causal scale stream : IO (dQ x dK x dV)
 // The triple is returned as the nested pair (dQ, (dK, dV)), Lean's representation of a x b x c.
 lean_object* lean_tyr_gpu_flash_attn_bwd(uint64_t B, uint64_t H, uint64_t N, uint64_t D,

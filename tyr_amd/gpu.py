@@ -67,20 +67,34 @@ def device_info(device: int = 0) -> dict:
             "clock_mhz": clk.value, "hbm_bytes": hbm.value}
 
 
-def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, stream=None):
-    """O, LSE = flashAttnFwd q k v causal scale.  q,k,v bf16 [B,H,N,D] -> (bf16 [B,H,N,D], f32 [B,H,N])."""
+def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, window: int = 0, kv_lens=None,
+                   stream=None):
+    """O, LSE = flashAttnFwd q k v causal scale.
+
+    q bf16 [B,Hq,N,D]; k, v bf16 [B,Hkv,N,D] with Hq % Hkv == 0 (query head h reads kv head h / (Hq/Hkv));
+    ``window`` > 0 (causal only) lets query i see keys (i - window, i]; ``kv_lens`` (int32 [B] on the device)
+    masks the keys at or beyond each sequence's length.  -> (bf16 [B,Hq,N,D], f32 [B,Hq,N])."""
     for t, n in ((q, "q"), (k, "k"), (v, "v")):
         _check(t, n, torch.bfloat16, 4)
-    if k.shape != q.shape or v.shape != q.shape:
-        raise TyrGpuError("q, k, v must have the same shape [B, H, N, D]")
-    B, H, N, D = q.shape
+    B, Hq, N, D = q.shape
+    if k.shape != v.shape or k.shape[0] != B or k.shape[2] != N or k.shape[3] != D:
+        raise TyrGpuError("k, v must have shape [B, Hkv, N, D] matching q's B, N, D")
+    Hkv = k.shape[1]
+    if Hkv == 0 or Hq % Hkv != 0:
+        raise TyrGpuError("the number of query heads must be a multiple of the number of kv heads")
     if scale is None:
         scale = 1.0 / math.sqrt(D)
+    lens_ptr = None
+    if kv_lens is not None:
+        _check(kv_lens, "kvLens", torch.int32, 1)
+        if kv_lens.numel() != B:
+            raise TyrGpuError("kvLens must hold one length per sequence")
+        lens_ptr = kv_lens.data_ptr()
     o = torch.empty_like(q)
-    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
-    rc = _lib.load().tyr_hip_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                            lse.data_ptr(), B, H, N, D, int(bool(causal)), float(scale),
-                                            _stream(stream))
+    lse = torch.empty((B, Hq, N), dtype=torch.float32, device=q.device)
+    rc = _lib.load().tyr_hip_flash_attn_fwd_gqa(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                lse.data_ptr(), B, Hq, Hkv, N, D, int(bool(causal)), int(window),
+                                                lens_ptr, float(scale), _stream(stream))
     _raise(rc, "flashAttnFwd")
     return o, lse
 

@@ -43,6 +43,16 @@ def capabilities : Capabilities := {}
 opaque flashAttnFwd {B H N D : UInt64} (q k v : @& T #[B, H, N, D]) (causal : Bool) (scale : Float)
     (stream : CudaStream) : IO (T #[B, H, N, D] × T #[B, H, N])
 
+/-- Flash-attention forward with grouped queries (`k v` carry `Hkv` heads, query head `h` reads kv head
+    `h / (Hq/Hkv)`), a causal sliding window (`window = 0`: none) and per-sequence key lengths
+    (`kvLens : int32 [B]`, keys at or beyond them are masked). GPU twin of `nn.scaledDotProductAttentionGQA`,
+    `…GQAWindow` and (for prefix padding masks) `…GQAMask` (`cc/src/tyr.cpp:3913-4095`; callers
+    `Tyr/Model/Qwen/Attention.lean:138,274`, `Tyr/Model/Qwen3TTS/SpeechTokenizer.lean:591`). -/
+@[extern "lean_tyr_gpu_flash_attn_fwd_gqa"]
+opaque flashAttnFwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (kvLens : @& T #[B]) (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hq, N])
+
 /-- Flash-attention backward. `o` and `lse` are the results of `flashAttnFwd` for the same
     `q k v causal scale`; `dO` is the upstream gradient. Returns `(dQ, dK, dV)`, bf16, final
     (no per-tile partials to reduce on the host). Replaces `tkMhaH100BwdPrep2Block` +
