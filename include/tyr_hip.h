@@ -152,6 +152,20 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
                        uint64_t kv_stride, float scale, uint64_t num_splits,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Flash-attention backward for the forward of tyr_hip_flash_attn_fwd_gqa (same q, k, v, causal,
+ * window, kv_lens, scale; o and lse its outputs).  dq : bf16 [B, Hq, N, D]; dk, dv : bf16
+ * [B, Hkv, N, D], each summed over the Hq/Hkv query heads that read that kv head (the gradient of
+ * the reference's repeat_interleave, cc/src/tyr.cpp:3930-3936).  Rows of dk / dv at or beyond a
+ * sequence's length are written as zero.  workspace: tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D).
+ * Supported additionally: (Hq/Hkv) * N * D * 2 < 2^31.  tyr_hip_flash_attn_bwd is this call with
+ * Hkv = Hq, window = 0, kv_lens = NULL.
+ */
+int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, const void* o,
+                               const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* GQA decode with a per-sequence cache length and / or a sliding window.
  *
  * Decode-time (one query token) form of `lean_torch_sdpa_gqa_mask` (padding mask: the valid

@@ -48,6 +48,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_attn_fwd_f64.restype = None
         L.oracle_attn_fwd_f64_ex.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, i64, vp, f64]
         L.oracle_attn_fwd_f64_ex.restype = None
+        L.oracle_attn_bwd_f64_ex.argtypes = [vp] * 7 + [i64] * 5 + [ci, i64, vp, f64]
+        L.oracle_attn_bwd_f64_ex.restype = None
         L.oracle_attn_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
         L.oracle_attn_bwd_f64.restype = None
         L.oracle_attn_fwd_tiled.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f32, i64]
@@ -145,6 +147,20 @@ def attn_bwd_f64(q, k, v, d_o, causal: bool, scale: float):
     dq, dk, dv = (np.empty((B, H, N, D), np.float32) for _ in range(3))
     lib().oracle_attn_bwd_f64(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), B, H, N, D,
                               int(causal), float(scale))
+    return dq, dk, dv
+
+
+def attn_bwd_f64_ex(q, k, v, d_o, causal: bool, scale: float, window: int = 0, kv_lens=None):
+    """Double-precision attention backward with grouped queries, window and key lengths.
+    q, d_o uint16 [B,Hq,N,D]; k, v uint16 [B,Hkv,N,D] -> (dQ [B,Hq,N,D], dK, dV [B,Hkv,N,D]) f32."""
+    q, k, v, d_o = (_chk(t, np.uint16, n) for t, n in ((q, "q"), (k, "k"), (v, "v"), (d_o, "d_o")))
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    dq = np.empty((B, Hq, N, D), np.float32)
+    dk, dv = np.empty((B, Hkv, N, D), np.float32), np.empty((B, Hkv, N, D), np.float32)
+    lens = None if kv_lens is None else _chk(np.asarray(kv_lens, dtype=np.int32), np.int32, "kv_lens")
+    lib().oracle_attn_bwd_f64_ex(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), B, Hq, Hkv, N, D, int(causal),
+                                 int(window), None if lens is None else _p(lens), float(scale))
     return dq, dk, dv
 
 

@@ -25,6 +25,9 @@
  *                           dV = P^T dO, dK = scale dS^T Q, dQ = scale dS K), in
  *                           double; reference values as Examples/GPU/RunMhaH100.lean:56-64
  *                           takes them from autograd.
+ *   oracle_attn_bwd_f64_ex  the same with grouped queries (dK / dV summed over the query
+ *                           heads of a kv head: the gradient of repeat_interleave), window
+ *                           and prefix key lengths.
  *   oracle_gqa_decode       cc/src/tyr.cpp:4100-4133 (repeat_interleave mapping),
  *                           Tyr/GPU/Kernels/FlashAttn3.lean:535-624 (q-head packing),
  *                           split/merge algebra of Tyr/GPU/Kernels/RingAttn.lean
@@ -257,6 +260,76 @@ void oracle_attn_bwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v
         for (int64_t x = 0; x < N * D; ++x) {
             dk[bh * N * D + x] = (float)dka[x];
             dv[bh * N * D + x] = (float)dva[x];
+        }
+        free(dka); free(dva); free(p); free(dp); free(dqa);
+    }
+}
+
+/* Attention backward in double precision with grouped queries, sliding window and per-sequence
+ * key length (visibility rule of oracle_attn_fwd_f64_ex).  dq: f32 [B,Hq,N,D]; dk, dv: f32
+ * [B,Hkv,N,D], each the sum over the Hq/Hkv query heads that read that kv head (the gradient of
+ * repeat_interleave is that sum).  Rows without a visible key contribute nothing. */
+void oracle_attn_bwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                            const uint16_t* d_o, float* dq, float* dk, float* dv,
+                            int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                            int causal, int64_t window, const int32_t* kv_lens, double scale) {
+    const int64_t G = Hq / Hkv;
+    #pragma omp parallel for schedule(dynamic)
+    for (int64_t bk = 0; bk < B * Hkv; ++bk) {
+        const int64_t b = bk / Hkv, kvh = bk % Hkv;
+        const uint16_t* kh = k + bk * N * D;
+        const uint16_t* vh = v + bk * N * D;
+        int64_t len = kv_lens ? kv_lens[b] : N;
+        if (len > N) len = N;
+        if (len < 1) len = 1;
+        double* dka = (double*)calloc((size_t)(N * D), sizeof(double));
+        double* dva = (double*)calloc((size_t)(N * D), sizeof(double));
+        double* p = (double*)malloc(sizeof(double) * (size_t)N);
+        double* dp = (double*)malloc(sizeof(double) * (size_t)N);
+        double* dqa = (double*)malloc(sizeof(double) * (size_t)D);
+        for (int64_t hq = 0; hq < G; ++hq) {
+            const int64_t bh = b * Hq + kvh * G + hq;
+            const uint16_t* qh = q + bh * N * D;
+            const uint16_t* gh = d_o + bh * N * D;
+            for (int64_t i = 0; i < N; ++i) {
+                const int64_t jhi = causal ? (i + 1 < len ? i + 1 : len) : len;
+                const int64_t jlo = window > 0 ? (i - window + 1 > 0 ? i - window + 1 : 0) : 0;
+                for (int64_t d = 0; d < D; ++d) dqa[d] = 0.0;
+                if (jlo < jhi) {
+                    double m = -INFINITY;
+                    for (int64_t j = jlo; j < jhi; ++j) {
+                        double acc = 0.0;
+                        for (int64_t d = 0; d < D; ++d)
+                            acc += (double)bf16_to_f32(qh[i * D + d]) * (double)bf16_to_f32(kh[j * D + d]);
+                        p[j] = acc * scale;
+                        if (p[j] > m) m = p[j];
+                    }
+                    double l = 0.0;
+                    for (int64_t j = jlo; j < jhi; ++j) { p[j] = exp(p[j] - m); l += p[j]; }
+                    double delta = 0.0;
+                    for (int64_t j = jlo; j < jhi; ++j) {
+                        p[j] /= l;
+                        double acc = 0.0;
+                        for (int64_t d = 0; d < D; ++d)
+                            acc += (double)bf16_to_f32(gh[i * D + d]) * (double)bf16_to_f32(vh[j * D + d]);
+                        dp[j] = acc;
+                        delta += p[j] * acc;
+                    }
+                    for (int64_t j = jlo; j < jhi; ++j) {
+                        const double ds = p[j] * (dp[j] - delta) * scale;
+                        for (int64_t d = 0; d < D; ++d) {
+                            dqa[d] += ds * (double)bf16_to_f32(kh[j * D + d]);
+                            dka[j * D + d] += ds * (double)bf16_to_f32(qh[i * D + d]);
+                            dva[j * D + d] += p[j] * (double)bf16_to_f32(gh[i * D + d]);
+                        }
+                    }
+                }
+                for (int64_t d = 0; d < D; ++d) dq[(bh * N + i) * D + d] = (float)dqa[d];
+            }
+        }
+        for (int64_t x = 0; x < N * D; ++x) {
+            dk[bk * N * D + x] = (float)dka[x];
+            dv[bk * N * D + x] = (float)dva[x];
         }
         free(dka); free(dva); free(p); free(dp); free(dqa);
     }

@@ -75,6 +75,31 @@ def test_flash_attn_bwd_random_shapes(gpu, seed):
         check(got, want, (what, B, H, N, D, causal))
 
 
+@pytest.mark.parametrize("mode", ["gqa", "gqa_noncausal", "window", "lens", "lens_noncausal", "all"])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(2, 4, 2, 300, 128), (1, 8, 1, 200, 64), (8, 2, 1, 130, 128)])
+def test_flash_attn_bwd_grouped_window_lengths(gpu, B, Hq, Hkv, N, D, mode):
+    # the backward of tyr_hip_flash_attn_fwd_gqa: dK / dV summed over the query heads of a kv head
+    # (gradient of the reference's repeat_interleave), window and prefix key lengths as in the forward
+    q, g = lt.make_inputs(8100 + N, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(8101 + N, (B, Hkv, N, D), (B, Hkv, N, D))
+    sc = 1 / math.sqrt(D)
+    causal = "noncausal" not in mode
+    window = 70 if mode in ("window", "all") else 0
+    lens = ([N, 1, N // 2, 65, N, 3, N - 1, 128][:B]) if mode in ("lens", "lens_noncausal", "all") else None
+    lens_d = None if lens is None else torch.tensor(lens, dtype=torch.int32, device="cuda")
+    qd, kd, vd, gd = (t.cuda() for t in (q, k, v, g))
+    o, lse = gpu.flash_attn_fwd(qd, kd, vd, causal=causal, scale=sc, window=window, kv_lens=lens_d)
+    dq, dk, dv = gpu.flash_attn_bwd(qd, kd, vd, o, lse, gd, causal=causal, scale=sc, window=window, kv_lens=lens_d)
+    wq, wk, wv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), causal, sc, window=window, kv_lens=lens)
+    check(dq, wq, ("dq", mode))
+    check(dk, wk, ("dk", mode))
+    check(dv, wv, ("dv", mode))
+    if lens is not None:                              # no gradient reaches keys / values beyond a sequence's length
+        for b, n in enumerate(lens):
+            assert float(dk[b, :, n:].float().abs().max() if n < N else 0.0) == 0.0
+            assert float(dv[b, :, n:].float().abs().max() if n < N else 0.0) == 0.0
+
+
 def test_flash_attn_bwd_properties(gpu):
     # exact linearity in a power-of-two multiple of dO; bit-identical repeat runs (no atomics);
     # rows of dS sum to zero, hence sum_j dK[j] = scale * sum_i (sum_j dS[i,j]) Q[i] = 0.

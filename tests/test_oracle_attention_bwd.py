@@ -100,3 +100,47 @@ def test_bwd_invariants():
     p_last = torch.softmax(s, -1)[:, :, 0, -1]
     want = p_last[..., None] * g.double()[:, :, -1, :]
     np.testing.assert_allclose(dv[:, :, -1, :], want.numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("mode", ["gqa", "window", "lens", "all"])
+def test_bwd_ex_matches_autograd_of_the_libtorch_mask_sequences(mode):
+    # gradients of lean_torch_sdpa_gqa / _window / _mask taken by autograd (repeat_interleave's
+    # gradient sums dK / dV over the query heads of a kv head)
+    B, Hq, Hkv, N, D = 2, 4, 2, 50, 16
+    q, g = lt.make_inputs(61, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(62, (B, Hkv, N, D), (B, Hkv, N, D))
+    window = 9 if mode in ("window", "all") else 0
+    lens = [50, 13] if mode in ("lens", "all") else None
+    causal = mode != "lens"
+    dq, dk, dv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), causal, 0.25, window=window, kv_lens=lens)
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    n = N
+    row, col = torch.arange(n).unsqueeze(1), torch.arange(n).unsqueeze(0)
+    hidden = torch.zeros(B, 1, n, n, dtype=torch.bool)
+    if causal:
+        hidden = hidden | (col > row)
+    if window:
+        hidden = hidden | ((row - col) >= window)
+    if lens is not None:
+        hidden = hidden | (col[None, None] >= torch.tensor(lens).view(B, 1, 1, 1))
+    mask = torch.zeros(B, 1, n, n, dtype=torch.float64).masked_fill(hidden, float("-inf"))
+    kr, vr = k64.repeat_interleave(Hq // Hkv, 1), v64.repeat_interleave(Hq // Hkv, 1)
+    # rows that see no key would be NaN in torch; give them one dummy visible key and zero their upstream gradient
+    dead = hidden.all(-1, keepdim=True)
+    mask = torch.where(dead.expand_as(mask), torch.zeros_like(mask), mask)
+    out = torch.nn.functional.scaled_dot_product_attention(q64, kr, vr, mask, 0.0, False, scale=0.25)
+    gg = g.double() * (~dead).double()
+    out.backward(gg)
+    dq_ref = q64.grad
+    np.testing.assert_allclose(dq, dq_ref.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dk, k64.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dv, v64.grad.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_bwd_ex_reduces_to_plain_backward():
+    B, H, N, D = 1, 3, 33, 16
+    q, k, v, g = rand4(71, B, H, N, D)
+    a = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), True, 0.3)
+    b = oracle.attn_bwd_f64(bits(q), bits(k), bits(v), bits(g), True, 0.3)
+    for x, y in zip(a, b):
+        np.testing.assert_allclose(x, y, rtol=1e-6, atol=1e-7)

@@ -122,23 +122,36 @@ int tyr_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const vo
                            const void* d_o, const float* lse, void* dq, void* dk, void* dv,
                            uint64_t B, uint64_t H, uint64_t N, uint64_t D, int causal, float scale,
                            void* workspace, size_t workspace_bytes, void* stream) {
+    return tyr_hip_flash_attn_bwd_gqa(q, k, v, o, d_o, lse, dq, dk, dv, B, H, H, N, D, causal, 0, nullptr, scale,
+                                      workspace, workspace_bytes, stream);
+}
+
+int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, const void* o,
+                               const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return TYR_HIP_ERR_NULL_POINTER;
-    if (B == 0 || H == 0 || N == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (B == 0 || Hq == 0 || Hkv == 0 || N == 0 || D == 0 || Hq % Hkv != 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return TYR_HIP_ERR_UNSUPPORTED;
+    if (window > 0 && !causal) return TYR_HIP_ERR_UNSUPPORTED;
     if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
-    if (!fits_int(N) || !fits_int(B * H) || B * H > (uint64_t)INT_MAX / ((N + 127) / 128))
+    if (!fits_int(N) || !fits_int(B * Hq) || B * Hq > (uint64_t)INT_MAX / ((N + 127) / 128))
         return TYR_HIP_ERR_BAD_SHAPE;
-    if (N * D * 2 >= ((uint64_t)1 << 31)) return TYR_HIP_ERR_UNSUPPORTED;   // 32-bit offsets inside one head
+    // 32-bit offsets inside the G query heads of one kv head (and inside their pairs)
+    if ((Hq / Hkv) * N * D * 2 >= ((uint64_t)1 << 31)) return TYR_HIP_ERR_UNSUPPORTED;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||
         !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
         return TYR_HIP_ERR_MISALIGNED;
     if (reinterpret_cast<uintptr_t>(lse) & 3u) return TYR_HIP_ERR_MISALIGNED;
-    const size_t need = tyr_hip_flash_attn_bwd_workspace_bytes(B, H, N, D);
+    if (kv_lens && (reinterpret_cast<uintptr_t>(kv_lens) & 3u)) return TYR_HIP_ERR_MISALIGNED;
+    const size_t need = tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D);
     if (!workspace || workspace_bytes < need) return TYR_HIP_ERR_WORKSPACE;
     if (!aligned16(workspace)) return TYR_HIP_ERR_MISALIGNED;
-    const int rc = tyr::launch_flash_attn_bwd(q, k, v, o, d_o, lse, dq, dk, dv, (int)B, (int)H, (int)N,
-                                              (int)D, causal != 0, scale, workspace,
-                                              static_cast<hipStream_t>(stream));
+    const int rc = tyr::launch_flash_attn_bwd(q, k, v, o, d_o, lse, dq, dk, dv, (int)B, (int)Hq, (int)Hkv, (int)N,
+                                              (int)D, causal != 0,
+                                              (int)(window > (uint64_t)INT_MAX ? INT_MAX : window), kv_lens, scale,
+                                              workspace, static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }
 

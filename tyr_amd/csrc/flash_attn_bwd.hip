@@ -35,6 +35,7 @@
 // LDS tiles are row-major with 16-byte chunks XOR-swizzled by a function of the row that is
 // conflict-free both for row fragments (16-byte reads, lane = row) and for transposed fragments
 // (ds_read_b64_tr_b16 over 4 rows x 64 bytes per lane-group pair).
+#include <limits.h>
 #include <type_traits>
 
 #include "common.hpp"
@@ -117,12 +118,14 @@ __device__ __forceinline__ void store_transposed_bf16(const f32x16 (&acc)[D / 32
 
 // ------------------------------------------------------------------------------------------
 // dQ (and the (lse2, delta) pairs)
-template <int D, bool CAUSAL>
+// EXT adds the per-sequence key length and the sliding window (same rule as the forward kernel);
+// G = query heads per kv head.
+template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     const uint16_t* __restrict__ O, const uint16_t* __restrict__ dO, const float* __restrict__ LSE,
     uint16_t* __restrict__ dQ, float2* __restrict__ stats, int BH, int N, int ntq, float scale,
-    float scale_log2) {
+    float scale_log2, int Hq, int G, int window, const int* __restrict__ kv_lens) {
     using namespace fab;
     using C = CfgQ<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -131,27 +134,36 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r = lane & 31, g = lane >> 5;
 
-    int bh, qt;
+    int bh, qt, kvbh;
     {
         const int id = blockIdx.x;
+        const int ngroups = BH / G;              // B * Hkv: the unit dealt to an XCD shares one K / V
         int tr;
-        if ((BH & 7) == 0) {
+        if ((ngroups & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
-            bh = (slot / ntq) * 8 + xcd;
-            tr = slot % ntq;
+            const int per_group = G * ntq;
+            kvbh = (slot / per_group) * 8 + xcd;
+            const int within = slot % per_group;
+            tr = within / G;
+            const int hkv = Hq / G;
+            bh = (kvbh / hkv) * Hq + (kvbh % hkv) * G + within % G;
         } else {
             bh = id / ntq;
             tr = id % ntq;
+            kvbh = (bh / Hq) * (Hq / G) + (bh % Hq) / G;
         }
         qt = CAUSAL ? ntq - 1 - tr : tr;
     }
     const int q0 = qt * C::BM;
     const int qw0 = q0 + w * 32;
     const size_t head_off = (size_t)bh * N * D;
-    const uint16_t* Kh = Kp + head_off;
-    const uint16_t* Vh = Vp + head_off;
-    const int kv_end = CAUSAL ? min(N, q0 + C::BM) : N;
-    const int nkv = (kv_end + C::BN - 1) / C::BN;
+    const uint16_t* Kh = Kp + (size_t)kvbh * N * D;
+    const uint16_t* Vh = Vp + (size_t)kvbh * N * D;
+    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    const int kv_end = CAUSAL ? min(Nk, q0 + C::BM) : Nk;
+    const int nkv_abs = (kv_end + C::BN - 1) / C::BN;
+    const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / C::BN, nkv_abs - 1) : 0;
+    const int nkv = nkv_abs - jbase;             // tiles are numbered from jbase below
     const int qpos = qw0 + r;
 
     // ---- this wave's Q^T and dO^T fragments (lane = query row, columns 16i + 8g + [0,8)),
@@ -172,6 +184,7 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
         }
         delta = part + xor32(part);
         lse2 = LSE[(size_t)bh * N + qrow] * LOG2E;
+        if (EXT && lse2 == -INFINITY) lse2 = INFINITY;      // a row that saw no key: every probability is 0
         if (g == 0) {
             const size_t npad = (size_t)ntq * C::BM;
             stats[(size_t)bh * npad + qpos] = qpos < N ? make_float2(lse2, delta) : make_float2(INFINITY, 0.0f);
@@ -225,16 +238,16 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) dq[i][e] = 0.0f;
 
-    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / C::BN + 1) : nkv;
+    const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / C::BN + 1 - jbase) : nkv;
 
-    issue_kv(0, 0);
+    issue_kv(0, jbase * C::BN);
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(qf[i]); pin_registers(dof[i]); }
     wait_vmcnt0();
     __syncthreads();
 
     for (int j = 0; j < nkv; ++j) {
-        const int j0 = j * C::BN;
+        const int j0 = (jbase + j) * C::BN;
         if (j + 1 < nkv) issue_kv((j + 1) & 1, j0 + C::BN);
         if (j < nkv_w) {
             const unsigned char* Kt = lds + (j & 1) * C::TILE;
@@ -262,16 +275,18 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             }
             // mask (diagonal tiles, ragged tail): register e of sub-tile T is kv row
             // j0 + 32T + 8(e/4) + 4g + e%4
-            const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > N);
+            const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
             if (need_mask) {
-                const int lim = CAUSAL ? min(qpos, N - 1) : N - 1;
+                const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;
+                const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;
                 const int base = j0 + 4 * g;
 #pragma unroll
                 for (int T = 0; T < 2; ++T)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        if (kv > lim) s[T][e] = -INFINITY;
+                        if (kv > lim || (EXT && kv < low)) s[T][e] = -INFINITY;
                     }
             }
             // dS^T = P^T o (dP^T - delta), packed into column-operand slots (group c = 2T + sh
@@ -312,11 +327,15 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
 
 // ------------------------------------------------------------------------------------------
 // dK, dV
-template <int D, bool CAUSAL>
+// BHkv = batch * kv heads; the G query heads of a kv head are walked one after the other and
+// accumulate into the same dK / dV (the gradient of repeat_interleave).  EXT as above; with it
+// every step carries the mask instructions.
+template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     const uint16_t* __restrict__ dO, const float2* __restrict__ stats, uint16_t* __restrict__ dK,
-    uint16_t* __restrict__ dV, int BH, int N, int ntk, int npad, float scale, float scale_log2) {
+    uint16_t* __restrict__ dV, int BHkv, int N, int ntk, int npad, float scale, float scale_log2,
+    int Hq, int G, int window, const int* __restrict__ kv_lens) {
     using namespace fab;
     using C = CfgK<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -325,10 +344,10 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r = lane & 31, g = lane >> 5;
 
-    int bh, kt;
+    int bh, kt;                           // bh indexes (batch, kv head)
     {
         const int id = blockIdx.x;
-        if ((BH & 7) == 0) {
+        if ((BHkv & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
             bh = (slot / ntk) * 8 + xcd;
             kt = slot % ntk;              // causal: key tile 0 meets every query tile, so heavy first
@@ -340,7 +359,10 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const int n0 = kt * C::BNK;
     const int nw0 = n0 + w * 32;
     const int kvpos = nw0 + r;
-    const size_t head_off = (size_t)bh * N * D;
+    const size_t head_off = (size_t)bh * N * D;                       // of K, V, dK, dV
+    const int hkv = Hq / G;
+    const size_t qh0 = (size_t)(bh / hkv) * Hq + (size_t)(bh % hkv) * G;   // first query head of the group
+    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / hkv])) : N;
 
     // ---- this wave's K and V rows as column operands (lane = key row, columns 16i + 8g + [0,8))
     bf16x8 kf[C::KSTEPS], vf[C::KSTEPS];
@@ -354,11 +376,14 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     }
 
     // ---- Q / dO / pair tile loaders
+    // The G query heads of the group are adjacent in memory: one buffer covers them, a head is a
+    // scalar offset.  (Rows past N of a head then alias the next head's first rows instead of
+    // reading as zero; their pairs are (+inf, 0), so their probabilities are exactly 0 either way.)
     const uint32_t head_bytes = (uint32_t)N * D * 2u;
-    const u32x4 q_rsrc = make_raw_rsrc(Q + head_off, head_bytes);
-    const u32x4 do_rsrc = make_raw_rsrc(dO + head_off, head_bytes);
+    const u32x4 q_rsrc = make_raw_rsrc(Q + qh0 * N * D, head_bytes * (uint32_t)G);
+    const u32x4 do_rsrc = make_raw_rsrc(dO + qh0 * N * D, head_bytes * (uint32_t)G);
     const uint32_t stat_bytes = (uint32_t)npad * 8u;
-    const u32x4 st_rsrc = make_raw_rsrc(stats + (size_t)bh * npad, stat_bytes);
+    const u32x4 st_rsrc = make_raw_rsrc(stats + qh0 * npad, stat_bytes * (uint32_t)G);
     constexpr int ROWS_PER_INST = 1024 / C::ROW;
     int g_voff[C::PT];
 #pragma unroll
@@ -371,11 +396,15 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const int nq = (N + C::BQ - 1) / C::BQ;
     // Tiles past the end are requested at an offset beyond the buffer (they read as zero), so that
     // every iteration issues the same number of loads and the wait count below stays constant.
+    const int jq0 = CAUSAL ? n0 / C::BQ : 0;
+    // with a window the last query that sees a key of this block is n0 + 127 + window - 1
+    const int jq_end = (EXT && window > 0) ? min(nq, (n0 + C::BNK + window - 2) / C::BQ + 1) : nq;
+    int hq = 0;                                      // query head of the group being walked
     auto issue_tile = [&](int stage, int jq) {
         const uint32_t dst = wave_dst + (uint32_t)stage * C::STAGE;
-        const bool live = jq < nq;
-        const int soff = live ? jq * C::BQ * C::ROW : (int)head_bytes;
-        const int ssoff = live ? jq * C::BQ * 8 : (int)stat_bytes;
+        const bool live = jq < jq_end;
+        const int soff = live ? hq * (int)head_bytes + jq * C::BQ * C::ROW : (int)(head_bytes * (uint32_t)G);
+        const int ssoff = live ? (hq * npad + jq * C::BQ) * 8 : (int)(stat_bytes * (uint32_t)G);
 #pragma unroll
         for (int m = 0; m < C::PT; ++m) {
             load_global_to_lds_16(q_rsrc, dst + m * 1024, g_voff[m], soff);
@@ -406,8 +435,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) { dk[i][e] = 0.0f; dv[i][e] = 0.0f; }
 
-    const int jq0 = CAUSAL ? n0 / C::BQ : 0;
-    const int ntile = nq - jq0;
+    const int ntile = jq_end - jq0;
     const int nsub = 2 * ntile;                       // 32-row sub-tiles, numbered from the block's first tile
     // First sub-tile with a visible (query, key) pair for this wave.  Causal: the block's first
     // tile starts at query n0 and the wave's keys at n0 + 32w, so sub-tile w is the wave's diagonal
@@ -493,8 +521,12 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
                 for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
                 if (need_mask) {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x)
-                        if (kvpos > qs0 + 8 * (2 * sh + h) + 4 * g + x) p[x] = 0.0f;
+                    for (int x = 0; x < 4; ++x) {
+                        const int qrow = qs0 + 8 * (2 * sh + h) + 4 * g + x;
+                        const bool hidden = (CAUSAL && kvpos > qrow) ||
+                                            (EXT && ((window > 0 && qrow - kvpos >= window) || kvpos >= Nk));
+                        if (hidden) p[x] = 0.0f;
+                    }
                 }
 #pragma unroll
                 for (int x = 0; x < 4; ++x) ds[x] = p[x] * (dp[8 * sh + 4 * h + x] - dl[x]);
@@ -565,6 +597,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
 
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) { pin_registers(kf[i]); pin_registers(vf[i]); }
+    for (hq = 0; hq < G; ++hq) {
     issue_tile(0, jq0);
     issue_tile(1, jq0 + 1);
     issue_tile(2, jq0 + 2);
@@ -581,7 +614,8 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         }
     };
     using std::integral_constant;
-    using MaskedT = integral_constant<bool, CAUSAL>;
+    using MaskedT = integral_constant<bool, CAUSAL || EXT>;
+    using SteadyMaskedT = integral_constant<bool, EXT>;
     const int qbase = jq0 * C::BQ;
     // Scores ping-pong between two register sets by the parity of u (no copies).
     f32x16 sA, dpA, sB, dpB;
@@ -603,7 +637,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     case K:                                                                                                  \
         if (u >= nsub) goto pipeline_done;                                                                   \
         tile_boundary(u);                                                                                    \
-        step(std::false_type{}, std::false_type{}, integral_constant<int, (K) / 2>{},                        \
+        step(SteadyMaskedT{}, std::false_type{}, integral_constant<int, (K) / 2>{},                          \
              integral_constant<int, (K) % 2>{}, qbase + 32 * u, CS, CD, NS, ND);                             \
         ++u;                                                                                                 \
         [[fallthrough]];
@@ -622,8 +656,9 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     }
 pipeline_done:
 #undef TYR_STEP
-    wait_vmcnt0();
+    wait_vmcnt0();                                   // drain before the next head reuses the stages
     __syncthreads();
+    }
 
     unsigned char* scratch = lds + w * (32 * (D * 2 + 16));
     store_transposed_bf16<D>(dv, 1.0f, scratch, dV + head_off + (size_t)nw0 * D, N - nw0, lane);
@@ -636,13 +671,14 @@ size_t flash_attn_bwd_workspace_bytes(int B, int H, int N) {
 }
 
 int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
-                          const float* lse, void* dq, void* dk, void* dv, int B, int H, int N, int D,
-                          int causal, float scale, void* workspace, hipStream_t stream) {
+                          const float* lse, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int N, int D,
+                          int causal, int window, const int* kv_lens, float scale, void* workspace,
+                          hipStream_t stream) {
     using namespace fab;
-    const int BH = B * H;
+    const int BH = B * Hq, BHkv = B * Hkv, G = Hq / Hkv;
     const int ntq = (N + 127) / 128;
     const int npad = ntq * 128;
-    dim3 grid((unsigned)(BH * ntq)), block(THREADS);
+    dim3 grid_q((unsigned)(BH * ntq)), grid_k((unsigned)(BHkv * ntq)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
     auto Kp = static_cast<const uint16_t*>(k);
@@ -650,24 +686,31 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     auto Op = static_cast<const uint16_t*>(o);
     auto dOp = static_cast<const uint16_t*>(d_o);
     auto st = static_cast<float2*>(workspace);
-#define TYR_FAB_LAUNCH(DD, CC)                                                                        \
+    const bool ext = window > 0 || kv_lens != nullptr;
+#define TYR_FAB_LAUNCH(DD, CC, EE)                                                                    \
     do {                                                                                              \
         static const hipError_t a1 = hipFuncSetAttribute(                                             \
-            reinterpret_cast<const void*>(&flash_attn_bwd_dq_kernel<DD, CC>),                         \
+            reinterpret_cast<const void*>(&flash_attn_bwd_dq_kernel<DD, CC, EE>),                     \
             hipFuncAttributeMaxDynamicSharedMemorySize, CfgQ<DD>::LDS);                               \
         static const hipError_t a2 = hipFuncSetAttribute(                                             \
-            reinterpret_cast<const void*>(&flash_attn_bwd_dkv_kernel<DD, CC>),                        \
+            reinterpret_cast<const void*>(&flash_attn_bwd_dkv_kernel<DD, CC, EE>),                    \
             hipFuncAttributeMaxDynamicSharedMemorySize, CfgK<DD>::LDS);                               \
         if (a1 != hipSuccess || a2 != hipSuccess) return -1;                                          \
-        hipLaunchKernelGGL((flash_attn_bwd_dq_kernel<DD, CC>), grid, block, CfgQ<DD>::LDS, stream,    \
+        hipLaunchKernelGGL((flash_attn_bwd_dq_kernel<DD, CC, EE>), grid_q, block, CfgQ<DD>::LDS, stream, \
                            Qp, Kp, Vp, Op, dOp, lse, static_cast<uint16_t*>(dq), st, BH, N, ntq,      \
-                           scale, scale_log2);                                                        \
-        hipLaunchKernelGGL((flash_attn_bwd_dkv_kernel<DD, CC>), grid, block, CfgK<DD>::LDS, stream,   \
+                           scale, scale_log2, Hq, G, window, kv_lens);                                \
+        hipLaunchKernelGGL((flash_attn_bwd_dkv_kernel<DD, CC, EE>), grid_k, block, CfgK<DD>::LDS, stream, \
                            Qp, Kp, Vp, dOp, st, static_cast<uint16_t*>(dk),                           \
-                           static_cast<uint16_t*>(dv), BH, N, ntq, npad, scale, scale_log2);          \
+                           static_cast<uint16_t*>(dv), BHkv, N, ntq, npad, scale, scale_log2, Hq, G,  \
+                           window, kv_lens);                                                          \
     } while (0)
-    if (D == 128) { if (causal) TYR_FAB_LAUNCH(128, true); else TYR_FAB_LAUNCH(128, false); }
-    else          { if (causal) TYR_FAB_LAUNCH(64, true);  else TYR_FAB_LAUNCH(64, false); }
+#define TYR_FAB_PICK(DD)                                                                              \
+    do {                                                                                              \
+        if (ext) { if (causal) TYR_FAB_LAUNCH(DD, true, true); else TYR_FAB_LAUNCH(DD, false, true); }    \
+        else     { if (causal) TYR_FAB_LAUNCH(DD, true, false); else TYR_FAB_LAUNCH(DD, false, false); }  \
+    } while (0)
+    if (D == 128) TYR_FAB_PICK(128); else TYR_FAB_PICK(64);
+#undef TYR_FAB_PICK
 #undef TYR_FAB_LAUNCH
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -99,29 +99,42 @@ def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, win
     return o, lse
 
 
-def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | None = None, stream=None):
+def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | None = None, window: int = 0,
+                   kv_lens=None, stream=None):
     """dQ, dK, dV = flashAttnBwd q k v o lse dO causal scale.
 
-    q, k, v, o, d_o bf16 [B,H,N,D]; lse f32 [B,H,N]; o and lse as returned by flash_attn_fwd for
-    the same q, k, v, causal and scale.  Returns three bf16 [B,H,N,D] tensors."""
+    q, o, d_o bf16 [B,Hq,N,D]; k, v bf16 [B,Hkv,N,D]; lse f32 [B,Hq,N]; o and lse as returned by
+    flash_attn_fwd for the same q, k, v, causal, scale, window and kv_lens.  Returns dQ [B,Hq,N,D] and
+    dK, dV [B,Hkv,N,D] (summed over the query heads of each kv head), bf16."""
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "dO")):
         _check(t, n, torch.bfloat16, 4)
-        if t.shape != q.shape:
-            raise TyrGpuError("q, k, v, o, dO must have the same shape [B, H, N, D]")
+    if o.shape != q.shape or d_o.shape != q.shape or k.shape != v.shape:
+        raise TyrGpuError("q, o, dO must have the same shape [B, Hq, N, D] and k, v the same shape [B, Hkv, N, D]")
     _check(lse, "lse", torch.float32, 3)
-    B, H, N, D = q.shape
-    if tuple(lse.shape) != (B, H, N):
+    B, Hq, N, D = q.shape
+    if k.shape[0] != B or k.shape[2] != N or k.shape[3] != D:
+        raise TyrGpuError("q, k, v, o, dO must have the same shape [B, H, N, D] (k, v may have fewer heads)")
+    Hkv = k.shape[1]
+    if Hkv == 0 or Hq % Hkv != 0:
+        raise TyrGpuError("the number of query heads must be a multiple of the number of kv heads")
+    if tuple(lse.shape) != (B, Hq, N):
         raise TyrGpuError("lse must have shape [B, H, N]")
     if scale is None:
         scale = 1.0 / math.sqrt(D)
+    lens_ptr = None
+    if kv_lens is not None:
+        _check(kv_lens, "kvLens", torch.int32, 1)
+        if kv_lens.numel() != B:
+            raise TyrGpuError("kvLens must hold one length per sequence")
+        lens_ptr = kv_lens.data_ptr()
     lib = _lib.load()
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
-    nbytes = lib.tyr_hip_flash_attn_bwd_workspace_bytes(B, H, N, D)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(k)
+    nbytes = lib.tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D)
     ws = torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=q.device)
-    rc = lib.tyr_hip_flash_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
-                                    lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D,
-                                    int(bool(causal)), float(scale), ws.data_ptr(), ws.numel(),
-                                    _stream(stream))
+    rc = lib.tyr_hip_flash_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
+                                        lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, N, D,
+                                        int(bool(causal)), int(window), lens_ptr, float(scale), ws.data_ptr(),
+                                        ws.numel(), _stream(stream))
     _raise(rc, "flashAttnBwd")
     return dq, dk, dv
 

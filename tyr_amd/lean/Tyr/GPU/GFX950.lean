@@ -64,6 +64,15 @@ opaque flashAttnBwd {B H N D : UInt64} (q k v o : @& T #[B, H, N, D]) (lse : @& 
     (dO : @& T #[B, H, N, D]) (causal : Bool) (scale : Float) (stream : CudaStream)
     : IO (T #[B, H, N, D] × T #[B, H, N, D] × T #[B, H, N, D])
 
+/-- Backward of `flashAttnFwdGQA` (same `q k v kvLens causal window scale`; `o lse` its results).
+    Returns `(dQ : [B,Hq,N,D], dK, dV : [B,Hkv,N,D])`; `dK dV` are summed over the query heads that read
+    each kv head, which is the gradient of the reference's `repeat_interleave` (`cc/src/tyr.cpp:3930-3936`). -/
+@[extern "lean_tyr_gpu_flash_attn_bwd_gqa"]
+opaque flashAttnBwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (o : @& T #[B, Hq, N, D]) (lse : @& T #[B, Hq, N]) (dO : @& T #[B, Hq, N, D]) (kvLens : @& T #[B])
+    (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
+
 /-- GQA decode attention, one query token per sequence, split-KV with an LSE combine pass.
     `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D = 128`,
     query head `h` reads kv head `h / (Hq/Hkv)`; `numSplits = 0` lets the library choose.
