@@ -141,7 +141,7 @@ int tyr_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const vo
  *   num_splits : KV chunks per (b, kv head); 0 = choose automatically.
  *   workspace  : device scratch of at least tyr_hip_gqa_decode_workspace_bytes(...) bytes,
  *                16-byte aligned; contents need not be initialised.
- * Supported: D == 128; 1 <= Hq/Hkv <= 16 with Hq % Hkv == 0; L >= 1; num_splits <= 64.
+ * Supported: D in {64, 128}; 1 <= Hq/Hkv <= 16 with Hq % Hkv == 0; L >= 1; num_splits <= 64.
  */
 size_t tyr_hip_gqa_decode_workspace_bytes(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L,
                                           uint64_t D, uint64_t num_splits);

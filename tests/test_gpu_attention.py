@@ -214,6 +214,26 @@ def test_gqa_decode_matches_oracle(gpu, B, Hq, Hkv, L, splits):
     assert max_abs(o.cpu().float(), ref) <= TOL
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,splits", [(2, 8, 2, 300, 0), (1, 4, 4, 33, 1), (3, 16, 1, 1000, 4), (1, 6, 2, 1, 1)])
+def test_gqa_decode_head_dim_64(gpu, B, Hq, Hkv, L, splits):
+    D = 64
+    q, = lt.make_inputs(450 + L, (B, Hq, 1, D))
+    k, v = lt.make_inputs(451 + L, (B, Hkv, L, D), (B, Hkv, L, D))
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits)
+    want_o, want_lse = oracle.gqa_decode(bits(q), bits(k), bits(v), sc, max(splits, 1))
+    assert max_abs(o.cpu().float(), from_bits(want_o).float()) <= TOL
+    assert max_abs(lse.cpu(), want_lse) <= 1e-3
+    ref = lt.sdpa_gqa_qkv(q.float(), k.float(), v.float(), False, True)
+    assert max_abs(o.cpu().float(), ref) <= TOL
+    # decode == last row of the causal prefill kernel at the same head dimension
+    if Hq == Hkv:
+        qf = torch.zeros(B, Hq, L, D, dtype=torch.bfloat16)
+        qf[:, :, -1:] = q
+        of, _ = gpu.flash_attn_fwd(qf.cuda(), k.cuda(), v.cuda(), causal=True, scale=sc)
+        assert max_abs(o.cpu().float(), of[:, :, -1:].cpu().float()) <= TOL
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_gqa_decode_random_shapes(gpu, seed):
     rng = np.random.default_rng(2000 + seed)

@@ -180,7 +180,7 @@ int tyr_hip_gqa_decode_varlen(const void* q, const void* k, const void* v, void*
     if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
     if (B == 0 || Hq == 0 || Hkv == 0 || L == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (Hq % Hkv != 0 || kv_stride < L) return TYR_HIP_ERR_BAD_SHAPE;
-    if (D != 128 || Hq / Hkv > 16 || num_splits > kMaxSplits) return TYR_HIP_ERR_UNSUPPORTED;
+    if ((D != 128 && D != 64) || Hq / Hkv > 16 || num_splits > kMaxSplits) return TYR_HIP_ERR_UNSUPPORTED;
     if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
     if (!fits_int(L) || !fits_int(B * Hq) || B * Hkv > 65535 || kv_stride > (uint64_t)INT_MAX)
         return TYR_HIP_ERR_BAD_SHAPE;

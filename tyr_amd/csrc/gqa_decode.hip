@@ -26,19 +26,22 @@
 namespace tyr {
 
 namespace dec {
-constexpr int STEP = 32, D = 128, QPAD = 16;
+constexpr int STEP = 32, QPAD = 16;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+template <int D>
 struct Buf {
-    u32x4 k[2][4];   // [T][i]: row 16T + x, d = 32i + 8g + [0,8)
-    u32x4 v[8];      // [p]  : row 16(p/4) + 4g + p%4, d = 8x + [0,8)
+    u32x4 k[2][D / 32];   // [T][i]: row 16T + x, d = 32i + 8g + [0,8)
+    u32x4 v[8];           // [p]  : row 16(p/4) + 4g + p%4, d = 8(x mod D/8) + [0,8)
 };
 }  // namespace dec
 
 // WAVES waves per workgroup share one split.  With a single split (S == 1) the workgroup writes
 // the final bf16 O and LSE itself and the second pass is skipped.
-template <int WAVES>
+// D = 64: a V row is 8 pieces, so lanes x >= 8 repeat the loads of lanes x - 8 (same cache lines, no
+// extra traffic) and rows 8..15 of every O^T MFMA tile (lane groups g >= 2) are unused.
+template <int WAVES, int D>
 __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     float* __restrict__ part_o, float* __restrict__ part_m, float* __restrict__ part_l,
@@ -70,11 +73,12 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const int nsteps = r1 > r0 ? (r1 - r0 + STEP - 1) / STEP : 0;
 
     // Q^T operand: column x = query head kvh*G + x (zero for x >= G)
-    bf16x8 qf[4];
+    constexpr int KI = D / 32;                  // MFMA k-steps of a score tile
+    bf16x8 qf[KI];
     {
         const uint16_t* qp = Q + ((size_t)b * Hq + (size_t)kvh * G + min(x, G - 1)) * D + g * 8;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < KI; ++i) {
             u32x4 v = ld_global_16(qp + i * 32);
             if (x >= G) v = u32x4{0, 0, 0, 0};
             qf[i] = __builtin_bit_cast(bf16x8, v);
@@ -86,28 +90,28 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     for (int j = 0; j < 8; ++j) oacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m2 = -INFINITY, lsum = 0.0f;
 
-    auto load = [&](Buf& bf, int row0) {
+    auto load = [&](Buf<D>& bf, int row0) {
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             const int row = min(row0 + 16 * T + x, L - 1);
             const uint16_t* kp = Kb + (size_t)row * D + g * 8;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) bf.k[T][i] = ld_global_16_nt(kp + i * 32);
+            for (int i = 0; i < KI; ++i) bf.k[T][i] = ld_global_16_nt(kp + i * 32);
         }
 #pragma unroll
         for (int p = 0; p < 8; ++p) {
             const int row = min(row0 + 16 * (p >> 2) + 4 * g + (p & 3), L - 1);
-            bf.v[p] = ld_global_16_nt(Vb + (size_t)row * D + x * 8);
+            bf.v[p] = ld_global_16_nt(Vb + (size_t)row * D + (x & (D / 8 - 1)) * 8);
         }
     };
 
-    auto compute = [&](const Buf& bf, int row0) {
+    auto compute = [&](const Buf<D>& bf, int row0) {
         f32x4 sacc[2];
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             sacc[T] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < KI; ++i)
                 sacc[T] = mfma_16x16x32_bf16(__builtin_bit_cast(bf16x8, bf.k[T][i]), qf[i], sacc[T]);
         }
         // register rr of sub-tile T is kv row row0 + 16T + 4g + rr
@@ -154,8 +158,8 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     };
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pin_registers(qf[i]);
-    Buf b0, b1;
+    for (int i = 0; i < KI; ++i) pin_registers(qf[i]);
+    Buf<D> b0, b1;
     if (nsteps > 0) load(b0, r0);
     for (int st = 0; st < nsteps; st += 2) {
         if (st + 1 < nsteps) load(b1, r0 + (st + 1) * STEP);
@@ -171,15 +175,15 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     float* sm = smem + WAVES * G * D;              // [WAVES][QPAD]
     float* sl = sm + WAVES * QPAD;                 // [WAVES][QPAD]
     const float ltot = sum_xor32(sum_xor16(lsum));
-    if (x < G) {
+    if (x < G && 32 * g < D) {
         float* dst = so + ((size_t)w * G + x) * D + 32 * g;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             *reinterpret_cast<f32x4*>(dst + 8 * rr) = f32x4{oacc[0][rr], oacc[1][rr], oacc[2][rr], oacc[3][rr]};
             *reinterpret_cast<f32x4*>(dst + 8 * rr + 4) = f32x4{oacc[4][rr], oacc[5][rr], oacc[6][rr], oacc[7][rr]};
         }
-        if (g == 0) { sm[w * QPAD + x] = m2; sl[w * QPAD + x] = ltot; }
     }
+    if (x < G && g == 0) { sm[w * QPAD + x] = m2; sl[w * QPAD + x] = ltot; }
     __syncthreads();
 
     for (int idx = t; idx < G * D; idx += THREADS) {
@@ -209,7 +213,8 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
 }
 
 // Second pass: one workgroup of D threads per (batch, query head).
-__global__ __launch_bounds__(dec::D) void gqa_decode_combine_kernel(
+template <int D>
+__global__ __launch_bounds__(D) void gqa_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_m, const float* __restrict__ part_l,
     uint16_t* __restrict__ O, float* __restrict__ LSE, int S) {
     using namespace dec;
@@ -239,7 +244,6 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
                       int Hq, int Hkv, int L, int D, int64_t kv_stride, float scale, int num_splits,
                       void* workspace, const int* kv_lens, int window, hipStream_t stream) {
     using namespace dec;
-    (void)D;
     constexpr int WAVES = 8;
     const int G = Hq / Hkv;
     const int S = num_splits;
@@ -250,26 +254,32 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
     wchunk = (wchunk + STEP - 1) / STEP * STEP;
 
     float* part_o = static_cast<float*>(workspace);
-    float* part_m = part_o + (size_t)B * Hq * S * dec::D;
+    float* part_m = part_o + (size_t)B * Hq * S * D;
     float* part_l = part_m + (size_t)B * Hq * S;
 
-    const size_t lds = (size_t)(WAVES * G * dec::D + 2 * WAVES * QPAD) * sizeof(float);
+    const size_t lds = (size_t)(WAVES * G * D + 2 * WAVES * QPAD) * sizeof(float);
     dim3 grid((unsigned)S, (unsigned)(B * Hkv)), block(64 * WAVES);
-    static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&gqa_decode_split_kernel<WAVES>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, (WAVES * QPAD * dec::D + 2 * WAVES * QPAD) * (int)sizeof(float));
-    if (attr != hipSuccess) return -1;
-    hipLaunchKernelGGL(gqa_decode_split_kernel<WAVES>, grid, block, lds, stream,
-                       static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k),
-                       static_cast<const uint16_t*>(v), part_o, part_m, part_l,
-                       static_cast<uint16_t*>(o), lse, Hq, Hkv, G, L, (long)kv_stride, S, chunk, wchunk,
-                       scale * LOG2E, kv_lens, window);
-    if (hipGetLastError() != hipSuccess) return -1;
-    if (S > 1) {
-        hipLaunchKernelGGL(gqa_decode_combine_kernel, dim3((unsigned)(B * Hq)), dim3(dec::D), 0, stream,
-                           part_o, part_m, part_l, static_cast<uint16_t*>(o), lse, S);
-        if (hipGetLastError() != hipSuccess) return -1;
-    }
+#define TYR_DEC_LAUNCH(DD)                                                                           \
+    do {                                                                                             \
+        static const hipError_t attr = hipFuncSetAttribute(                                          \
+            reinterpret_cast<const void*>(&gqa_decode_split_kernel<WAVES, DD>),                      \
+            hipFuncAttributeMaxDynamicSharedMemorySize,                                              \
+            (WAVES * QPAD * DD + 2 * WAVES * QPAD) * (int)sizeof(float));                            \
+        if (attr != hipSuccess) return -1;                                                           \
+        hipLaunchKernelGGL((gqa_decode_split_kernel<WAVES, DD>), grid, block, lds, stream,           \
+                           static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k),         \
+                           static_cast<const uint16_t*>(v), part_o, part_m, part_l,                  \
+                           static_cast<uint16_t*>(o), lse, Hq, Hkv, G, L, (long)kv_stride, S, chunk, \
+                           wchunk, scale * LOG2E, kv_lens, window);                                  \
+        if (hipGetLastError() != hipSuccess) return -1;                                              \
+        if (S > 1) {                                                                                 \
+            hipLaunchKernelGGL(gqa_decode_combine_kernel<DD>, dim3((unsigned)(B * Hq)), dim3(DD), 0, \
+                               stream, part_o, part_m, part_l, static_cast<uint16_t*>(o), lse, S);   \
+            if (hipGetLastError() != hipSuccess) return -1;                                          \
+        }                                                                                            \
+    } while (0)
+    if (D == 128) TYR_DEC_LAUNCH(128); else TYR_DEC_LAUNCH(64);
+#undef TYR_DEC_LAUNCH
     return 0;
 }
 

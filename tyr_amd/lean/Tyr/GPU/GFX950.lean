@@ -74,7 +74,7 @@ opaque flashAttnBwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : 
     : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
 
 /-- GQA decode attention, one query token per sequence, split-KV with an LSE combine pass.
-    `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D = 128`,
+    `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D ∈ {64, 128}`,
     query head `h` reads kv head `h / (Hq/Hkv)`; `numSplits = 0` lets the library choose.
     GPU twin of `nn.scaledDotProductAttentionGQAQKV` with `is_causal = false`
     (`Tyr/Torch.lean:1070-1082`, caller `Tyr/Model/Qwen/Attention.lean:199-200`). -/
