@@ -71,7 +71,7 @@ template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2,
-    int Hq, int G, int window, const int* __restrict__ kv_lens) {
+    int Hq, int G, int window, const int* __restrict__ kv_lens, int pair) {
     using namespace fa;
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -85,26 +85,30 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // are issued first.
     // With grouped queries (G > 1) the unit dealt to an XCD is a (batch, kv head) group: its G
     // query heads times ntq tiles share one K/V; the G heads of a tile are adjacent.
-    int bh, qt, kvbh;
+    // With `pair` (causal) a workgroup handles query tile ntq-1-tr and then tile tr: every
+    // workgroup does the same amount of work and there are half as many of them to start.
+    const int ntr = pair ? (ntq + 1) / 2 : ntq;  // tile ranks per head
+    int bh, tr, kvbh;
     {
         const int id = blockIdx.x;
         const int ngroups = BH / G;              // B * Hkv
-        int tr;
         if ((ngroups & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
-            const int per_group = G * ntq;
+            const int per_group = G * ntr;
             kvbh = (slot / per_group) * 8 + xcd;
             const int within = slot % per_group;
             tr = within / G;
             const int hkv = Hq / G;
             bh = (kvbh / hkv) * Hq + (kvbh % hkv) * G + within % G;
         } else {
-            bh = id / ntq;
-            tr = id % ntq;
+            bh = id / ntr;
+            tr = id % ntr;
             kvbh = (bh / Hq) * (Hq / G) + (bh % Hq) / G;
         }
-        qt = CAUSAL ? ntq - 1 - tr : tr;
     }
+    const int npass = (pair && ntq - 1 - tr != tr) ? 2 : 1;
+    for (int pass = 0; pass < npass; ++pass) {
+    const int qt = CAUSAL ? (pass == 0 ? ntq - 1 - tr : tr) : tr;
     const int q0 = qt * BM;
     const int qw0 = q0 + w * 32;                 // first query row of this wave
     const size_t head_off = (size_t)bh * N * D;
@@ -372,6 +376,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         }
     }
     if (qpos < N && LSE != nullptr && g == 0) LSE[(size_t)bh * N + qpos] = logf(ltot) + m2 * LN2;
+    __syncthreads();                             // the scratch is read; the stages may be refilled
+    }
 }
 
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
@@ -381,13 +387,14 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
     const int BH = B * Hq;
     const int G = Hq / Hkv;
     const int ntq = (N + BM - 1) / BM;
-    dim3 grid((unsigned)(BH * ntq)), block(THREADS);
+    const bool ext = window > 0 || kv_lens != nullptr;
+    const int pair = (causal && !ext && ntq > 1) ? 1 : 0;
+    dim3 grid((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
     auto Kp = static_cast<const uint16_t*>(k);
     auto Vp = static_cast<const uint16_t*>(v);
     auto Op = static_cast<uint16_t*>(o);
-    const bool ext = window > 0 || kv_lens != nullptr;
 #define TYR_FA_LAUNCH(DD, CC, EE)                                                                \
     do {                                                                                         \
         static const hipError_t attr = hipFuncSetAttribute(                                      \
@@ -395,7 +402,7 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DD>::LDS);                           \
         if (attr != hipSuccess) return -1;                                                       \
         hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC, EE>), grid, block, Cfg<DD>::LDS, stream, \
-                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens);  \
+                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens, pair); \
     } while (0)
 #define TYR_FA_PICK(DD)                                                                          \
     do {                                                                                         \
