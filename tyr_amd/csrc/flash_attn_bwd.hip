@@ -125,7 +125,7 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     const uint16_t* __restrict__ O, const uint16_t* __restrict__ dO, const float* __restrict__ LSE,
     uint16_t* __restrict__ dQ, float2* __restrict__ stats, int BH, int N, int ntq, float scale,
-    float scale_log2, int Hq, int G, int window, const int* __restrict__ kv_lens) {
+    float scale_log2, int Hq, int G, int window, const int* __restrict__ kv_lens, int pair) {
     using namespace fab;
     using C = CfgQ<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -134,26 +134,30 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r = lane & 31, g = lane >> 5;
 
-    int bh, qt, kvbh;
+    // With `pair` (causal) a workgroup handles query tile ntq-1-tr and then tile tr (equal work
+    // for every workgroup, half as many of them).
+    const int ntr = pair ? (ntq + 1) / 2 : ntq;
+    int bh, tr, kvbh;
     {
         const int id = blockIdx.x;
         const int ngroups = BH / G;              // B * Hkv: the unit dealt to an XCD shares one K / V
-        int tr;
         if ((ngroups & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
-            const int per_group = G * ntq;
+            const int per_group = G * ntr;
             kvbh = (slot / per_group) * 8 + xcd;
             const int within = slot % per_group;
             tr = within / G;
             const int hkv = Hq / G;
             bh = (kvbh / hkv) * Hq + (kvbh % hkv) * G + within % G;
         } else {
-            bh = id / ntq;
-            tr = id % ntq;
+            bh = id / ntr;
+            tr = id % ntr;
             kvbh = (bh / Hq) * (Hq / G) + (bh % Hq) / G;
         }
-        qt = CAUSAL ? ntq - 1 - tr : tr;
     }
+    const int npass = (pair && ntq - 1 - tr != tr) ? 2 : 1;
+    for (int pass = 0; pass < npass; ++pass) {
+    const int qt = CAUSAL ? (pass == 0 ? ntq - 1 - tr : tr) : tr;
     const int q0 = qt * C::BM;
     const int qw0 = q0 + w * 32;
     const size_t head_off = (size_t)bh * N * D;
@@ -323,6 +327,8 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
 
     store_transposed_bf16<D>(dq, scale, lds + w * (32 * (D * 2 + 16)), dQ + head_off + (size_t)qw0 * D,
                              N - qw0, lane);
+    __syncthreads();                             // the scratch is read; the stages may be refilled
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -678,7 +684,9 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     const int BH = B * Hq, BHkv = B * Hkv, G = Hq / Hkv;
     const int ntq = (N + 127) / 128;
     const int npad = ntq * 128;
-    dim3 grid_q((unsigned)(BH * ntq)), grid_k((unsigned)(BHkv * ntq)), block(THREADS);
+    const bool ext = window > 0 || kv_lens != nullptr;
+    const int pair = (causal && !ext && ntq > 1) ? 1 : 0;
+    dim3 grid_q((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), grid_k((unsigned)(BHkv * ntq)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
     auto Kp = static_cast<const uint16_t*>(k);
@@ -686,7 +694,6 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     auto Op = static_cast<const uint16_t*>(o);
     auto dOp = static_cast<const uint16_t*>(d_o);
     auto st = static_cast<float2*>(workspace);
-    const bool ext = window > 0 || kv_lens != nullptr;
 #define TYR_FAB_LAUNCH(DD, CC, EE)                                                                    \
     do {                                                                                              \
         static const hipError_t a1 = hipFuncSetAttribute(                                             \
@@ -698,7 +705,7 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
         if (a1 != hipSuccess || a2 != hipSuccess) return -1;                                          \
         hipLaunchKernelGGL((flash_attn_bwd_dq_kernel<DD, CC, EE>), grid_q, block, CfgQ<DD>::LDS, stream, \
                            Qp, Kp, Vp, Op, dOp, lse, static_cast<uint16_t*>(dq), st, BH, N, ntq,      \
-                           scale, scale_log2, Hq, G, window, kv_lens);                                \
+                           scale, scale_log2, Hq, G, window, kv_lens, pair);                          \
         hipLaunchKernelGGL((flash_attn_bwd_dkv_kernel<DD, CC, EE>), grid_k, block, CfgK<DD>::LDS, stream, \
                            Qp, Kp, Vp, dOp, st, static_cast<uint16_t*>(dk),                           \
                            static_cast<uint16_t*>(dv), BHkv, N, ntq, npad, scale, scale_log2, Hq, G,  \
