@@ -107,6 +107,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         }
     }
     const int npass = (pair && ntq - 1 - tr != tr) ? 2 : 1;
+    bf16x8 qf[C::KSTEPS];                        // Q^T fragments: lane holds row qw0+r, columns 16i + 8g + [0,8)
+    bool preloaded = false;                      // this tile's K(0), K(1) and Q were requested by the previous one
     for (int pass = 0; pass < npass; ++pass) {
     const int qt = CAUSAL ? (pass == 0 ? ntq - 1 - tr : tr) : tr;
     const int q0 = qt * BM;
@@ -124,15 +126,14 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / BN, nkv_abs - 1) : 0;   // first tile any row sees
     const int nkv = nkv_abs - jbase;             // tiles are numbered from jbase below
 
-    // ---- Q^T fragments: lane holds row qw0+r, columns 16i + 8g + [0,8)
-    bf16x8 qf[C::KSTEPS];
-    {
-        const int qrow = min(qw0 + r, N - 1);
+    auto load_q = [&](int first_row) {
+        const int qrow = min(first_row + r, N - 1);
         const uint16_t* qp = Qh + (size_t)qrow * D + g * 8;
 #pragma unroll
         for (int i = 0; i < C::KSTEPS; ++i)
             qf[i] = __builtin_bit_cast(bf16x8, ld_global_16(qp + i * 16));
-    }
+    };
+    if (!preloaded) load_q(qw0);
 
     // ---- K/V tile loaders.  Buffer loads: the per-thread byte offset inside a tile is fixed, the
     // tile start is a scalar offset, and rows at or beyond N read as zero (they are masked below).
@@ -192,6 +193,10 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         }
     }
     const int qpos = qw0 + r;
+    // The second tile of a pair starts under the end of the first: its K(0), K(1) are requested
+    // in the first tile's last two steps (stage parity needs an even tile count), its Q rows
+    // before the first tile's output is written.
+    const bool overlap_next = pass + 1 < npass && (nkv & 1) == 0;
     // number of kv tiles that intersect this wave's visible region
     const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / BN + 1 - jbase) : nkv;
 
@@ -213,9 +218,13 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     };
 
     // ---- prologue: K(0), V(0), K(1) in flight; S(0) computed on its own
-    issue_k(0, jbase * BN);
-    issue_v(0, jbase * BN);
-    if (nkv > 1) issue_k(1, (jbase + 1) * BN);
+    if (!preloaded) {
+        issue_k(0, jbase * BN);
+        issue_v(0, jbase * BN);
+        if (nkv > 1) issue_k(1, (jbase + 1) * BN);
+    } else {
+        issue_v(0, 0);                           // K(0), K(1) and Q were requested by the first tile
+    }
 #pragma unroll
     for (int i = 0; i < C::KSTEPS; ++i) pin_registers(qf[i]);
     wait_vmcnt0();
@@ -240,7 +249,9 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         const int j0 = (jbase + j) * BN;
         // The two requests are issued apart (K here, V after the row-max reduction) so the waves of
         // a CU do not all queue on the texture path at once.
-        if (j + 2 < nkv) issue_k(j & 1, j0 + 2 * BN);
+        // In the last two steps of the first tile of a pair the freed K stages take K(0) and K(1) of
+        // the second tile (a full one, >= 2 kv tiles, starting from key 0).
+        if (j + 2 < nkv || overlap_next) issue_k(j & 1, j + 2 < nkv ? j0 + 2 * BN : (j + 2 - nkv) * BN);
         if (j >= nkv_w && j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
 
         if (j < nkv_w) {
@@ -349,13 +360,19 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     }
 
     // ---- finalize: O /= l, LSE = ln l + m.  The wave's 32 x D block of O goes through a private LDS
-    // scratch (all K/V stages are dead after the last barrier) so that global stores are 16 bytes
-    // per lane along rows.
+    // scratch in the V stages (dead after the last barrier; the K stages may already be filling for
+    // the second tile of a pair) so that global stores are 16 bytes per lane along rows.  Rows are
+    // unpadded; 16-byte chunks are XOR-swizzled by row.
+    if (overlap_next) load_q(tr * BM + w * 32);
     const float ltot = sum_xor32(lsum);
     const float inv = (!EXT || ltot > 0.0f) ? 1.0f / ltot : 0.0f;    // EXT: a row that saw no key gives 0
     {
-        constexpr int SROW = D * 2 + 16;
-        unsigned char* scratch = lds + w * (32 * SROW);
+        constexpr int SROW = D * 2;
+        constexpr int CH = D / 8;                   // 16-byte chunks per row
+        auto s_swz = [](int row) { return (D == 128 ? row : (row >> 1)) & (CH - 1); };
+        unsigned char* scratch = lds + C::V_BASE + w * (32 * SROW);
+        int wr_swz = s_swz(r) * 16;
+        asm volatile("" : "+v"(wr_swz));            // keeps the 16 swizzled addresses out of the main loop's registers
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
 #pragma unroll
@@ -363,20 +380,20 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
                 u32x2 v;
                 v.x = pack_bf16(oacc[dt][4 * q4 + 0] * inv, oacc[dt][4 * q4 + 1] * inv);
                 v.y = pack_bf16(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv);
-                *reinterpret_cast<u32x2*>(scratch + r * SROW + (dt * 32 + q4 * 8 + g * 4) * 2) = v;
+                *reinterpret_cast<u32x2*>(scratch + r * SROW + (((dt * 4 + q4) * 16) ^ wr_swz) + g * 8) = v;
             }
         }
-        constexpr int CH = D / 8;                   // 16-byte chunks per row
         constexpr int RPI = 64 / CH;                // rows per store instruction
 #pragma unroll
         for (int k = 0; k < 32 / RPI; ++k) {
             const int row = lane / CH + RPI * k;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * SROW + (lane % CH) * 16);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * SROW + ((lane % CH) ^ s_swz(row)) * 16);
             if (qw0 + row < N) st_global_16(O + head_off + (size_t)(qw0 + row) * D + (lane % CH) * 8, v);
         }
     }
     if (qpos < N && LSE != nullptr && g == 0) LSE[(size_t)bh * N + qpos] = logf(ltot) + m2 * LN2;
     __syncthreads();                             // the scratch is read; the stages may be refilled
+    preloaded = overlap_next;
     }
 }
 
