@@ -568,17 +568,9 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     // With one wave per SIMD nothing else hides LDS latency and every instruction of the wave costs
     // issue time, so fragments are requested a phase ahead and addresses cost no instructions.
     // Past the last sub-tile the "next" reads hit a stage without live data; their results are dropped.
-    auto step = [&](auto masked, auto first, auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc, f32x16& sn,
-                    f32x16& dpn) {
+    auto step = [&](auto masked, auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc, f32x16& sn, f32x16& dpn) {
         constexpr int STG = decltype(stg)::value, T = decltype(sub)::value;
-        using Stg1 = std::integral_constant<int, T == 0 ? STG : ((STG + 1) & 3)>;     // stage of u+1
-        using Sub1 = std::integral_constant<int, 1 - T>;
         using Stg2 = std::integral_constant<int, (STG + 1) & 3>;                        // stage of u+2
-        if (decltype(first)::value) {                 // the wave's first sub-tile: nothing was prepared
-            read_rows(stg, sub, rq, rd);
-            scores(rq, rd, sc, dpc);
-            read_rows(Stg1{}, Sub1{}, rq, rd);
-        }
         bf16x8 dot0[C::DT], qt0[C::DT], dot1[C::DT], qt1[C::DT];
         read_transposed(stg, 2 * T, dot0, qt0);
         f32x4 st[8];
@@ -598,6 +590,23 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             dv[dt] = mfma_32x32x16_bf16(dot1[dt], pf[1], dv[dt]);
             dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf[1], dk[dt]);
         }
+    };
+    // What a step expects of the step before it, for the wave's first sub-tile: its scores, and the
+    // row fragments of the sub-tile after it.  Without EXT the only partially masked sub-tile of a
+    // causal wave is this one (its diagonal): hidden scores become -inf here, which the steps turn
+    // into P = 0 and dS = 0 like any other score, so they carry no mask instructions.
+    auto first_scores = [&](auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc) {
+        constexpr int STG = decltype(stg)::value, T = decltype(sub)::value;
+        using Stg1 = std::integral_constant<int, T == 0 ? STG : ((STG + 1) & 3)>;     // stage of u+1
+        using Sub1 = std::integral_constant<int, 1 - T>;
+        read_rows(stg, sub, rq, rd);
+        scores(rq, rd, sc, dpc);
+        if (CAUSAL && !EXT) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (kvpos > qs0 + 8 * (e >> 2) + 4 * g + (e & 3)) sc[e] = -INFINITY;
+        }
+        read_rows(Stg1{}, Sub1{}, rq, rd);
     };
 #undef TYR_STG
 
@@ -620,30 +629,27 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         }
     };
     using std::integral_constant;
-    using MaskedT = integral_constant<bool, CAUSAL || EXT>;
-    using SteadyMaskedT = integral_constant<bool, EXT>;
+    using MaskedT = integral_constant<bool, EXT>;
     const int qbase = jq0 * C::BQ;
     // Scores ping-pong between two register sets by the parity of u (no copies).
     f32x16 sA, dpA, sB, dpB;
     int u = 0;
     for (; u < u0 && u < nsub; ++u) tile_boundary(u);           // sub-tiles above the wave's diagonal
     if (u < nsub) {
-        tile_boundary(u);
-        // u = u0 < 4: stage u0 / 2, sub-tile u0 % 2
+        // u = u0 < 4: stage u0 / 2, sub-tile u0 % 2; even sub-tiles keep their scores in sA / dpA
         switch (u) {
-            case 0:  step(MaskedT{}, std::true_type{}, integral_constant<int, 0>{}, integral_constant<int, 0>{}, qbase, sA, dpA, sB, dpB); break;
-            case 1:  step(MaskedT{}, std::true_type{}, integral_constant<int, 0>{}, integral_constant<int, 1>{}, qbase + 32, sB, dpB, sA, dpA); break;
-            case 2:  step(MaskedT{}, std::true_type{}, integral_constant<int, 1>{}, integral_constant<int, 0>{}, qbase + 64, sA, dpA, sB, dpB); break;
-            default: step(MaskedT{}, std::true_type{}, integral_constant<int, 1>{}, integral_constant<int, 1>{}, qbase + 96, sB, dpB, sA, dpA); break;
+            case 0:  first_scores(integral_constant<int, 0>{}, integral_constant<int, 0>{}, qbase, sA, dpA); break;
+            case 1:  first_scores(integral_constant<int, 0>{}, integral_constant<int, 1>{}, qbase + 32, sB, dpB); break;
+            case 2:  first_scores(integral_constant<int, 1>{}, integral_constant<int, 0>{}, qbase + 64, sA, dpA); break;
+            default: first_scores(integral_constant<int, 1>{}, integral_constant<int, 1>{}, qbase + 96, sB, dpB); break;
         }
-        ++u;
     }
-    // steady state, unrolled over the 8 (stage, sub-tile) combinations; entered at u % 8
+    // the pipeline, unrolled over the 8 (stage, sub-tile) combinations; entered at u % 8
 #define TYR_STEP(K, CS, CD, NS, ND)                                                                          \
     case K:                                                                                                  \
         if (u >= nsub) goto pipeline_done;                                                                   \
         tile_boundary(u);                                                                                    \
-        step(SteadyMaskedT{}, std::false_type{}, integral_constant<int, (K) / 2>{},                          \
+        step(MaskedT{}, integral_constant<int, (K) / 2>{},                                                   \
              integral_constant<int, (K) % 2>{}, qbase + 32 * u, CS, CD, NS, ND);                             \
         ++u;                                                                                                 \
         [[fallthrough]];
