@@ -55,7 +55,7 @@ def test_host_validation_needs_no_gpu():
     assert L.tyr_hip_flash_attn_fwd(p, p, p + 8, p, None, 1, 1, 16, 128, 1, 0.1, None) == MISAL
     assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 6, 4, 16, 128, 16, 0.1, 1, p, 1 << 20, None) == SHAPE   # Hq % Hkv
     assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 8, 2, 16, 128, 8, 0.1, 1, p, 1 << 20, None) == SHAPE   # stride < L
-    assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 8, 2, 16, 64, 16, 0.1, 1, p, 1 << 20, None) == UNSUP
+    assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 8, 2, 16, 96, 16, 0.1, 1, p, 1 << 20, None) == UNSUP
     assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 8, 2, 16, 128, 16, 0.1, 1, None, 0, None) == WS
     assert L.tyr_hip_gqa_decode(p, p, p, p, None, 1, 8, 2, 16, 128, 16, 0.1, 1, p, 64, None) == WS
     assert L.tyr_hip_gqa_decode_workspace_bytes(2, 8, 2, 1000, 128, 4) == 2 * 8 * 4 * 130 * 4

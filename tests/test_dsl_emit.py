@@ -1,0 +1,181 @@
+"""The tile DSL on CPU: the IR mirrors the reference's statement set, the builder lowers the
+reference's end-to-end kernels to the expected statement sequences, the emitter prints the expected
+gfx950 calls (the same style of substring goldens as Tyr/GPU/Codegen/Tests.lean:31-431), register-vector
+layouts are inferred, NVIDIA-only statements are refused, and the emitted translation unit compiles
+with hipcc for gfx950 (cross-compilation, no GPU)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from tyr_amd import dsl
+from tyr_amd.dsl import build as dsl_build
+from tyr_amd.dsl import kernels
+from tyr_amd.dsl.ir import KSTMT_FIELDS, VarId, stmt, walk
+
+REFERENCE_KSTMT = """declRT declST declRV declSV declSemaphore declGPtr declKVal load store loadAsync storeAsync storeAdd
+storeAddAsync storeMinAsync prefetch tmaExpect tmaLoad tmaStore loadGlobal storeGlobal loadGlobalAsync storeGlobalAsync
+storeGlobalAdd layoutDim loadVecGlobal storeVecGlobal storeVecGlobalAdd loadVecGlobalCoord storeVecGlobalCoord
+storeVecGlobalAddCoord loadScalarGlobal storeScalarGlobal multimemLoadReduce multimemStore multimemRed mma mm mmaFence
+mmaCommitGroup mmaAsyncWait tcgen05Mma cpAsyncLoad tmaLoadAsync unary binary ternary scalarMul scalarAdd broadcast
+binaryBroadcast reduce reduceAccum cumsum cumprod outer swapLayout transpose convert mask sliceRows sliceCols concatCols
+sync arrive arriveAndWait namedBarrierSync namedBarrierArrive warpGroupIdx electOneSync fenceViewAsyncShared
+fenceProxyAsync semaphore forLoop forLoopVal ifStmt ifWarpGroup comment getBlockIdx getThreadIdx constInt constFloat
+scalarUnary scalarCompare scalarBinary scalarSelect vecIota vecFillScalar raw""".split()
+
+
+def test_ir_has_every_reference_constructor():
+    # the constructor list of Tyr/GPU/Codegen/IR.lean:50-189, in order
+    assert list(KSTMT_FIELDS) == REFERENCE_KSTMT
+
+
+def test_stmt_checks_constructor_and_arity():
+    with pytest.raises(ValueError):
+        stmt("loadTile", VarId(0), VarId(1))
+    with pytest.raises(ValueError):
+        stmt("mma", "AB", VarId(0), VarId(1))
+    s = stmt("mma", "ABt", VarId(3), VarId(0), VarId(1), VarId(3))
+    assert (s.trans, s.dst, s.a, s.b, s.c) == ("ABt", VarId(3), VarId(0), VarId(1), VarId(3))
+
+
+def ops(kernel):
+    return [s.op for s in walk(kernel.body)]
+
+
+def test_copy_kernel_lowers_like_the_reference():
+    # Kernels/Copy.lean:16-26: comment, blockCoord2D (2 constInt + 2 getBlockIdx), allocRT, allocST, then
+    # loadGlobal, load, store, storeGlobal, sync
+    k = kernels.copy64x64()
+    assert [p.name for p in k.params] == ["input", "output"] and all(p.isPointer for p in k.params)
+    assert ops(k) == ["declGPtr", "declGPtr", "comment", "constInt", "constInt", "getBlockIdx", "getBlockIdx",
+                      "declRT", "declST", "loadGlobal", "load", "store", "storeGlobal", "sync"]
+    by = [s for s in k.body if s.op == "getBlockIdx"]
+    assert [s.axis for s in by] == [1, 0]                       # row = blockIdx.y, col = blockIdx.x
+
+
+def test_online_softmax_macro_expands_to_the_reference_sequence():
+    # Macros.lean:121-147: copyVec, rowMaxAccum, subVec, expVec, mulCol, mulVec, subCol, exp, rowSumAccum
+    k = kernels.tkFlashAttnFwd2BlockLse()
+    loop = next(s for s in k.body if s.op == "forLoop")
+    assert (loop.lo, loop.hi) == (0, 2)
+    body = list(loop.body)
+    i = next(n for n, s in enumerate(body) if s.op == "scalarMul")
+    assert body[i].scalar == 0.125
+    seq = [(s.op, s.args[0]) for s in body[i + 1:i + 10]]
+    assert seq == [("unary", "Copy"), ("reduceAccum", "Max"), ("binary", "Sub"), ("unary", "Exp"),
+                   ("binaryBroadcast", "Mul"), ("binary", "Mul"), ("binaryBroadcast", "Sub"), ("unary", "Exp"),
+                   ("reduceAccum", "Sum")]
+    assert [s.args[0] for s in body if s.op == "mma"] == ["ABt", "AB"]   # mmaT s q k s ; mma o p v o
+
+
+def test_emitted_text_goldens():
+    src = dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())
+    for needle in [
+        "__global__ __launch_bounds__(256) void tkFlashAttnFwd2BlockLse(gl<bf16> v0, gl<bf16> v1, gl<bf16> v2, "
+        "gl<bf16> v3, gl<float> v4, uint64_t v5, uint64_t v6)",
+        "rt<bf16, 64, 64, layout::col>",                       # v is a Col tile
+        "__shared__ st<bf16, 64, 64>",
+        "__shared__ sv<float, 64>",
+        "wave::mma_ABt(", "wave::mma_AB(",
+        "wave::scalar<op_mul>(", "0.125f);",
+        "wave::row_reduce<op_max>(", "wave::row_reduce<op_add>(",
+        "wave::col_broadcast<op_mul>(", "wave::col_broadcast<op_sub>(", "wave::col_broadcast<op_div>(",
+        "wave::unary<op_neg_infty>(", "wave::unary<op_log>(",
+        "for (int v", "wave::sync();",
+    ]:
+        assert needle in src, needle
+    # tile coordinates are scaled by the tile shape, as in EmitNew.lean:249-258
+    assert re.search(r"wave::load\(v\d+, v1, coord\{\(int\)v\d+, \(int\)v\d+, \(int\)v\d+ \* 64, \(int\)v\d+ \* 64\}\);", src)
+    # the vector store takes the row index as its unit coordinate (GlobalLayout.lean:343-349)
+    assert re.search(r"wave::store\(v4, v\d+, \(int\)v\d+\);", src)
+
+
+def test_register_vector_layouts_are_inferred():
+    # LayerNorm: statistics are reduced along rows and broadcast down columns (align); weight and bias
+    # are broadcast along rows (ortho), also through convertVec from their bf16 originals
+    k = kernels.tkFusedLayerNormResidual1024()
+    lay = dsl.infer_rv_layouts(k)
+    decl = [s for s in walk(k.body) if s.op == "declRV"]
+    assert len(decl) == 12
+    f32 = [s.v for s in decl if s.dtype == "Float32"]
+    bf = [s.v for s in decl if s.dtype == "BFloat16"]
+    assert [lay[v] for v in f32[:8]] == ["align"] * 8          # sum, sumSq, tmpSum, tmpSqSum, mean, meanSq, var, invStd
+    assert [lay[v] for v in f32[8:]] == ["ortho"] * 2          # weightF, biasF
+    assert [lay[v] for v in bf] == ["ortho"] * 2               # weightRV, biasRV
+    src = dsl.emit_kernel(k)
+    assert "rv<bf16, 64, vlayout::ortho>" in src and "rv<float, 64, vlayout::align>" in src
+    assert "wave::row_broadcast<op_mul>(" in src and "wave::row_broadcast<op_add>(" in src
+
+
+def test_conflicting_vector_use_is_an_error():
+    k = dsl.KernelBuilder("conflict")
+    t = k.allocRT("Float32", 64, 64)
+    v = k.allocRV("Float32", 64)
+    k.rowSum(v, t)          # align
+    k.mulRow(t, t, v)       # ortho
+    with pytest.raises(dsl.LayoutConflict, match="RV layout conflict for v1"):
+        dsl.emit_kernel(k.build())
+
+
+def test_nvidia_only_statements_are_refused_and_mma_bookkeeping_is_a_no_op():
+    k = dsl.KernelBuilder("tma")
+    a = k.allocST("BFloat16", 64, 64)
+    k.emit(stmt("prefetch", a.id))
+    with pytest.raises(dsl.UnsupportedStatement, match="prefetch"):
+        dsl.emit_kernel(k.build())
+    k = dsl.KernelBuilder("fence")
+    k.emit(stmt("mmaCommitGroup"))
+    k.emit(stmt("mmaAsyncWait", 0))
+    assert dsl.emit_kernel(k.build()).count("nothing to do") == 2
+
+
+def test_launcher_text():
+    tu = dsl.emit_translation_unit([kernels.rotaryFwd()])
+    assert ('extern "C" int tyr_launch_rotaryFwd(void* x_ptr, const int64_t* x_ptr_shape, int x_ptr_ndim, '
+            "void* sin_ptr") in tu
+    assert "uint64_t _seq_len, uint64_t _head_dim, uint64_t grid_x" in tu
+    assert "dim3(64 * waves)" in tu
+    # the Lean-facing wrapper keeps the reference's signature and messages (Attribute.lean:334-336, 344-352)
+    assert 'extern "C" lean_object* lean_launch_rotaryFwd(b_lean_obj_arg x_ptr, b_lean_obj_arg sin_ptr' in tu
+    for msg in ["x_ptr must be a CUDA tensor", "x_ptr must be contiguous", "x_ptr must have dim <= 4"]:
+        assert msg in tu
+
+
+def test_emitted_kernels_compile_for_gfx950(tmp_path):
+    src = dsl_build.emit_sources(str(tmp_path / "k.hip"))
+    cmd = [dsl_build.HIPCC] + dsl_build.HIPFLAGS + ["-I", dsl_build.CSRC, "-c", "--cuda-device-only", src, "-o",
+                                                    str(tmp_path / "k.o")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert os.path.getsize(tmp_path / "k.o") > 0
+
+
+def test_committed_header_matches_the_emitter_and_the_library_exports_it():
+    import ctypes
+    from tyr_amd.dsl import runtime
+    text = open(dsl_build.HEADER_PATH).read()
+    assert text == dsl_build.header_text(), "regenerate include/tyr_dsl_kernels.h: python -m tyr_amd.dsl.build"
+    names = re.findall(r"\bint (tyr_launch_\w+)\(", text)
+    assert names == [f"tyr_launch_{f().name}" for f in kernels.ALL]
+    L = runtime.load()
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_launcher_validates_on_the_host():
+    # no GPU needed: every call fails validation before the launch
+    import ctypes
+    from tyr_amd.dsl import runtime
+    L = runtime.load()
+    fn = L.tyr_launch_copy64x64
+    i64p, vp, u64 = ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p, ctypes.c_uint64
+    fn.argtypes = [vp, i64p, ctypes.c_int, vp, i64p, ctypes.c_int] + [u64] * 7 + [vp]
+    fn.restype = ctypes.c_int
+    shape = (ctypes.c_int64 * 4)(1, 1, 64, 64)
+    p = vp(0x1000)
+    assert fn(None, shape, 4, p, shape, 4, 1, 1, 1, 128, 1, 1, 0, None) == -2          # null tensor
+    assert fn(p, shape, 5, p, shape, 4, 1, 1, 1, 128, 1, 1, 0, None) == -2             # rank > 4
+    assert fn(p, shape, 4, p, shape, 4, 0, 1, 1, 128, 1, 1, 0, None) == -2             # empty grid
+    assert fn(p, shape, 4, p, shape, 4, 1, 1, 1, 0, 1, 1, 0, None) == -2               # empty block
+    assert fn(p, shape, 4, p, shape, 4, 1, 1, 1, 256, 1, 1, 0, None) == -2             # more warps than compiled for

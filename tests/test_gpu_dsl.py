@@ -1,0 +1,111 @@
+"""Emitted tile programs on the GPU against the CPU checker, with the inputs and bars of the
+reference's own runners: copy exact (Examples/GPU/RunCopy.lean:23-33), rotary allclose(1e-4, 1e-4)
+(RunRotary.lean:62-66), LayerNorm out allclose(5e-3, 5e-3) and residual allclose(1e-5, 1e-5)
+(RunLayerNorm.lean:66-71), attention O and LSE allclose(3e-2, 3e-2) on q,k,v [128,64], grid (1,2,1)
+(RunFlashAttn.lean:79-86) plus this build's own max-abs <= 2e-2, and the example GEMM against a float64
+product of the bf16 inputs (relative Frobenius <= 1e-2; the f32 result is far inside it)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import libtorch_path as lt
+from tests.util import bits, from_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from tyr_amd.dsl import kernels, runtime
+    runtime.load()
+    return kernels, runtime
+
+
+@pytest.mark.parametrize("block", [128, 32])
+@pytest.mark.parametrize("rows,cols,grid", [(64, 64, (1, 1, 1)), (128, 192, (3, 2, 1))])
+def test_copy64x64(rt, rows, cols, grid, block):
+    kernels, runtime = rt
+    g = torch.Generator().manual_seed(rows + cols)
+    x = torch.rand(1, 1, rows, cols, generator=g).cuda()
+    out = torch.zeros_like(x)
+    runtime.launch(kernels.copy64x64(), [x, out], grid=grid, block=(block, 1, 1))
+    torch.cuda.synchronize()
+    assert torch.equal(out, x)
+
+
+def test_rotaryFwd(rt):
+    kernels, runtime = rt
+    g = torch.Generator().manual_seed(7)
+    x = torch.rand(64, 64, generator=g)
+    cos, sin = lt.compute_rotary_freqs(64, 64)
+    want = oracle.rope(x.reshape(1, 64, 1, 64).numpy(), cos.numpy(), sin.numpy()).reshape(64, 64)
+    out = torch.zeros(64, 64).cuda()
+    runtime.launch(kernels.rotaryFwd(), [x.cuda(), sin.cuda().contiguous(), cos.cuda().contiguous(), out, 64, 64],
+                   grid=(1, 1, 1), block=(128, 1, 1))
+    torch.cuda.synchronize()
+    assert torch.allclose(out.cpu(), torch.from_numpy(want), rtol=1e-4, atol=1e-4)
+    assert float((out.cpu() - torch.from_numpy(want)).abs().max()) <= 1e-6
+
+
+@pytest.mark.parametrize("rows", [64, 192])
+def test_tkFusedLayerNormResidual1024(rt, rows):
+    kernels, runtime = rt
+    g = torch.Generator().manual_seed(rows)
+    x = torch.rand(1, rows, 1024, generator=g).bfloat16()
+    res = torch.rand(1, rows, 1024, generator=g).bfloat16()
+    w = torch.rand(1024, generator=g).bfloat16()
+    b = torch.rand(1024, generator=g).bfloat16()
+    want_out, want_resid = oracle.layernorm_residual(bits(x).reshape(rows, 1024), bits(res).reshape(rows, 1024),
+                                                     bits(w), bits(b), 1e-5)
+    out, out_resid = torch.zeros_like(x).cuda(), torch.zeros_like(x).cuda()
+    runtime.launch(kernels.tkFusedLayerNormResidual1024(), [x.cuda(), res.cuda(), w.cuda(), b.cuda(), out, out_resid],
+                   grid=(1, rows // 64, 1), block=(32, 1, 1))            # the runner's single-warp launch
+    torch.cuda.synchronize()
+    got_out, got_resid = out.cpu().float().reshape(rows, 1024), out_resid.cpu().float().reshape(rows, 1024)
+    assert torch.allclose(got_resid, from_bits(want_resid).float(), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(got_out, from_bits(want_out).float(), rtol=5e-3, atol=5e-3)
+
+
+@pytest.mark.parametrize("M,N", [(64, 64), (128, 192)])
+def test_simpleGemm(rt, M, N):
+    kernels, runtime = rt
+    K = 512                                                     # 8 K blocks of 64
+    a, b = lt.make_inputs(3, (M, K), (K, N), std=K ** -0.25)
+    c = torch.zeros(M, N).cuda()
+    runtime.launch(kernels.simpleGemm(), [a.cuda(), b.cuda(), c, M, N, K], grid=(N // 64, M // 64, 1),
+                   block=(128, 1, 1))
+    torch.cuda.synchronize()
+    want = a.double() @ b.double()
+    rel = float((c.cpu().double() - want).norm() / want.norm())
+    assert rel <= 1e-2 and rel <= 1e-5, rel
+
+
+def test_tkFlashAttnFwd2BlockLse(rt):
+    kernels, runtime = rt
+    q, k, v = lt.make_inputs(11, (128, 64), (128, 64), (128, 64))
+    o = torch.zeros(128, 64, dtype=torch.bfloat16).cuda()
+    lse = torch.zeros(128).cuda()
+    runtime.launch(kernels.tkFlashAttnFwd2BlockLse(), [q.cuda(), k.cuda(), v.cuda(), o, lse, 128, 64],
+                   grid=(1, 2, 1), block=(128, 1, 1))
+    torch.cuda.synchronize()
+    want_o, want_lse = oracle.attn_fwd_f64(bits(q).reshape(1, 1, 128, 64), bits(k).reshape(1, 1, 128, 64),
+                                           bits(v).reshape(1, 1, 128, 64), False, 0.125)
+    want_o, want_lse = torch.from_numpy(want_o).reshape(128, 64).float(), torch.from_numpy(want_lse).reshape(128).float()
+    assert torch.allclose(o.cpu().float(), want_o, rtol=3e-2, atol=3e-2)
+    assert torch.allclose(lse.cpu(), want_lse, rtol=3e-2, atol=3e-2)
+    assert float((o.cpu().float() - want_o).abs().max()) <= 2e-2
+    assert float((lse.cpu() - want_lse).abs().max()) <= 2e-2
+
+
+def test_launcher_rejects_bad_arguments(rt):
+    kernels, runtime = rt
+    x = torch.zeros(64, 64).cuda()
+    with pytest.raises(RuntimeError, match="input must be a CUDA tensor"):
+        runtime.launch(kernels.copy64x64(), [torch.zeros(64, 64), x])
+    with pytest.raises(RuntimeError, match="input must be contiguous"):
+        runtime.launch(kernels.copy64x64(), [torch.zeros(64, 128).cuda()[:, ::2], x])
+    with pytest.raises(RuntimeError, match="output must have dim <= 4"):
+        runtime.launch(kernels.copy64x64(), [x, torch.zeros(1, 1, 1, 64, 64).cuda()])
+    with pytest.raises(RuntimeError, match="invalid launch arguments"):
+        runtime.launch(kernels.copy64x64(), [x, x.clone()], block=(1024, 1, 1))

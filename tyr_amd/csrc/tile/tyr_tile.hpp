@@ -1,0 +1,526 @@
+// Wave-level tile vocabulary for gfx950 that programs emitted from the tile DSL are written in:
+// register tiles (rt), LDS tiles (st), register / LDS vectors (rv, sv), global layouts (gl) and
+// the operations of the DSL's statement set (Tyr/GPU/Codegen/IR.lean:50-189) on them.
+//
+// It plays the part the ThunderKittens headers play for the reference's emitter
+// (Tyr/GPU/Codegen/EmitNew.lean:207-330 prints `warp::load(...)`, `warp::mma_AB(...)`, ...), but it
+// is built around the 64-lane wave and the 32x32x16 bf16 MFMA, not around 32-lane warps:
+//
+//   * One wave owns a tile program.  A 32-thread "warp" of a reference launch maps to one wave.
+//   * Register tiles are grids of 32x32 blocks.  In a block of a ROW-layout tile lane
+//     l = (r = l % 32, g = l / 32) holds row r and the 16 columns 8q + 4g + x (q, x = 0..3) in slot
+//     4q + x.  A COL-layout tile is the transpose of that: lane holds column r and rows 8q + 4g + x.
+//   * That single layout is at once the MFMA accumulator layout (with the product issued
+//     transposed, so a lane owns a row) and a legal MFMA operand layout: an operand only has to
+//     agree with the other operand on which k sits in which (lane half, slot), and a ROW tile used
+//     as A[M,K] and a COL tile used as B[K,N] (or a ROW tile used as B^T[N,K]) agree by
+//     construction.  Products therefore read registers only, and exp(S) converted to bf16 is
+//     already the operand of the next product.
+//   * Row reductions are in-lane plus one exchange between the lane halves; their results live in
+//     ALIGN vectors (lane holds element 32b + r).  Column reductions and row-broadcast operands
+//     live in ORTHO vectors (lane holds elements 32c + 8q + 4g + x).  The emitter infers which.
+//
+// Everything is inline device code with compile-time indexing, so tiles stay in registers.
+#pragma once
+
+#include "../common.hpp"
+
+namespace tyr {
+namespace tile {
+
+typedef __bf16 bf16;
+
+enum class layout { row, col };
+enum class vlayout { align, ortho };
+
+struct coord {
+    int b, d, r, c;
+};
+
+// Row-major contiguous 4-D global tensor (batch, depth, rows, cols).
+template <typename T>
+struct gl {
+    T* ptr;
+    int nb, nd, nr, nc;
+    __device__ __forceinline__ T* at(int b, int d, int r, int c) const {
+        return ptr + ((((size_t)b * nd + d) * nr + r) * (size_t)nc + c);
+    }
+    __device__ __forceinline__ int batch() const { return nb; }
+    __device__ __forceinline__ int depth() const { return nd; }
+    __device__ __forceinline__ int rows() const { return nr; }
+    __device__ __forceinline__ int cols() const { return nc; }
+};
+
+template <typename T, int R, int C, layout L = layout::row>
+struct rt {
+    static_assert(R % 32 == 0 && C % 32 == 0, "register tiles are grids of 32x32 blocks");
+    typedef T dtype;
+    static constexpr int rows = R, cols = C, RB = R / 32, CB = C / 32;
+    static constexpr layout lay = L;
+    T data[RB][CB][16];
+};
+
+// LDS tile, row-major, rows padded by 16 bytes (32 lanes reading one column chunk of 32
+// consecutive rows then spread over the banks).
+template <typename T, int R, int C>
+struct st {
+    typedef T dtype;
+    static constexpr int rows = R, cols = C, pitch = C + 16 / (int)sizeof(T);
+    T data[R * pitch];
+    __device__ __forceinline__ T* at(int r, int c) { return data + r * pitch + c; }
+    __device__ __forceinline__ const T* at(int r, int c) const { return data + r * pitch + c; }
+};
+
+template <typename T, int N, vlayout V = vlayout::align>
+struct rv {
+    static_assert(N % 32 == 0, "register vectors are multiples of 32 elements");
+    typedef T dtype;
+    static constexpr int len = N, NB = N / 32;
+    static constexpr vlayout lay = V;
+    T data[NB][V == vlayout::align ? 1 : 16];
+};
+
+template <typename T, int N>
+struct sv {
+    typedef T dtype;
+    static constexpr int len = N;
+    T data[N];
+};
+
+namespace detail {
+__device__ __forceinline__ int lane() { return (int)(threadIdx.x & 63); }
+__device__ __forceinline__ int lr() { return lane() & 31; }
+__device__ __forceinline__ int lg() { return lane() >> 5; }
+// LDS traffic of one wave is ordered by the hardware; this keeps the compiler from moving
+// accesses across the point where other lanes' data is consumed.
+__device__ __forceinline__ void wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+template <typename T> __device__ __forceinline__ float to_f(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f(float x) { return (T)x; }
+// position of slot s of block (rb, cb) for the calling lane
+template <layout L> __device__ __forceinline__ int row_of(int rb, int s) {
+    return L == layout::row ? 32 * rb + lr() : 32 * rb + 8 * (s >> 2) + 4 * lg() + (s & 3);
+}
+template <layout L> __device__ __forceinline__ int col_of(int cb, int s) {
+    return L == layout::row ? 32 * cb + 8 * (s >> 2) + 4 * lg() + (s & 3) : 32 * cb + lr();
+}
+__device__ __forceinline__ float lane_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
+}  // namespace detail
+
+#define TYR_TILE_FOR_BLOCKS(RT)                                      \
+    _Pragma("unroll") for (int rb = 0; rb < RT::RB; ++rb)            \
+    _Pragma("unroll") for (int cb = 0; cb < RT::CB; ++cb)            \
+    _Pragma("unroll") for (int s = 0; s < 16; ++s)
+
+// ---------------------------------------------------------------- operation tags
+struct op_copy { static __device__ __forceinline__ float f(float x) { return x; } };
+struct op_zero { static __device__ __forceinline__ float f(float) { return 0.0f; } };
+struct op_one { static __device__ __forceinline__ float f(float) { return 1.0f; } };
+struct op_pos_infty { static __device__ __forceinline__ float f(float) { return INFINITY; } };
+struct op_neg_infty { static __device__ __forceinline__ float f(float) { return -INFINITY; } };
+struct op_exp { static __device__ __forceinline__ float f(float x) { return __expf(x); } };
+struct op_exp2 { static __device__ __forceinline__ float f(float x) { return exp2f(x); } };
+struct op_log { static __device__ __forceinline__ float f(float x) { return __logf(x); } };
+struct op_log2 { static __device__ __forceinline__ float f(float x) { return log2f(x); } };
+struct op_abs { static __device__ __forceinline__ float f(float x) { return fabsf(x); } };
+struct op_neg { static __device__ __forceinline__ float f(float x) { return -x; } };
+struct op_relu { static __device__ __forceinline__ float f(float x) { return fmaxf(x, 0.0f); } };
+struct op_sqrt { static __device__ __forceinline__ float f(float x) { return sqrtf(x); } };
+struct op_rsqrt { static __device__ __forceinline__ float f(float x) { return rsqrtf(x); } };
+struct op_recip { static __device__ __forceinline__ float f(float x) { return 1.0f / x; } };
+struct op_square { static __device__ __forceinline__ float f(float x) { return x * x; } };
+struct op_tanh { static __device__ __forceinline__ float f(float x) { return tanhf(x); } };
+struct op_sigmoid { static __device__ __forceinline__ float f(float x) { return 1.0f / (1.0f + __expf(-x)); } };
+struct op_silu { static __device__ __forceinline__ float f(float x) { return x / (1.0f + __expf(-x)); } };
+struct op_gelu {
+    static __device__ __forceinline__ float f(float x) {
+        return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+    }
+};
+struct op_sin { static __device__ __forceinline__ float f(float x) { return sinf(x); } };
+struct op_cos { static __device__ __forceinline__ float f(float x) { return cosf(x); } };
+
+struct op_add { static __device__ __forceinline__ float f(float a, float b) { return a + b; } };
+struct op_sub { static __device__ __forceinline__ float f(float a, float b) { return a - b; } };
+struct op_mul { static __device__ __forceinline__ float f(float a, float b) { return a * b; } };
+struct op_div { static __device__ __forceinline__ float f(float a, float b) { return a / b; } };
+struct op_max { static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); } };
+struct op_min { static __device__ __forceinline__ float f(float a, float b) { return fminf(a, b); } };
+
+
+// keep(i, j) decides which elements survive; the others take `fill`.
+struct keep_causal { static __device__ __forceinline__ bool f(int i, int j, int) { return j <= i; } };       // lower triangle incl. diagonal
+struct keep_causal_t { static __device__ __forceinline__ bool f(int i, int j, int) { return i <= j; } };
+struct keep_tril { static __device__ __forceinline__ bool f(int i, int j, int d) { return j <= i + d; } };
+struct keep_triu { static __device__ __forceinline__ bool f(int i, int j, int d) { return j >= i + d; } };
+struct keep_right_fill { static __device__ __forceinline__ bool f(int, int j, int d) { return j < d; } };      // columns >= d filled
+struct keep_left_fill { static __device__ __forceinline__ bool f(int, int j, int d) { return j >= d; } };      // columns < d filled
+struct keep_upper_fill { static __device__ __forceinline__ bool f(int i, int, int d) { return i >= d; } };     // rows < d filled
+struct keep_lower_fill { static __device__ __forceinline__ bool f(int i, int, int d) { return i < d; } };      // rows >= d filled
+
+namespace wave {
+using namespace detail;
+
+// ---------------------------------------------------------------- global <-> LDS
+template <typename T, int R, int C>
+__device__ __forceinline__ void load(st<T, R, C>& dst, const gl<T>& src, coord at) {
+    constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
+    static_assert(C % VEC == 0 && (R * CPR) % 64 == 0, "tile is not a whole number of 16-byte pieces per lane");
+#pragma unroll
+    for (int k = 0; k < R * CPR / 64; ++k) {
+        const int idx = lane() + 64 * k, r = idx / CPR, c = (idx % CPR) * VEC;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
+        *reinterpret_cast<u32x4*>(dst.at(r, c)) = v;
+    }
+    wave_fence();
+}
+template <typename T, int R, int C>
+__device__ __forceinline__ void store(const gl<T>& dst, const st<T, R, C>& src, coord at) {
+    constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
+    static_assert(C % VEC == 0 && (R * CPR) % 64 == 0, "tile is not a whole number of 16-byte pieces per lane");
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < R * CPR / 64; ++k) {
+        const int idx = lane() + 64 * k, r = idx / CPR, c = (idx % CPR) * VEC;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src.at(r, c));
+        *reinterpret_cast<u32x4*>(dst.at(at.b, at.d, at.r + r, at.c + c)) = v;
+    }
+}
+// vectors: element index = idx * N (the unit of a vector coordinate is the vector)
+template <typename T, int N>
+__device__ __forceinline__ void load(sv<T, N>& dst, const gl<T>& src, int idx) {
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) dst.data[lane() + 64 * k] = src.ptr[(size_t)idx * N + lane() + 64 * k];
+    wave_fence();
+}
+template <typename T, int N>
+__device__ __forceinline__ void store(const gl<T>& dst, const sv<T, N>& src, int idx) {
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) dst.ptr[(size_t)idx * N + lane() + 64 * k] = src.data[lane() + 64 * k];
+}
+template <typename T, int N>
+__device__ __forceinline__ void load(sv<T, N>& dst, const gl<T>& src, coord at) {
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) dst.data[lane() + 64 * k] = *src.at(at.b, at.d, at.r, at.c * N + lane() + 64 * k);
+    wave_fence();
+}
+template <typename T, int N>
+__device__ __forceinline__ void store(const gl<T>& dst, const sv<T, N>& src, coord at) {
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) *dst.at(at.b, at.d, at.r, at.c * N + lane() + 64 * k) = src.data[lane() + 64 * k];
+}
+
+// ---------------------------------------------------------------- LDS <-> registers
+template <typename T, int R, int C, layout L>
+__device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *src.at(row_of<L>(rb, s), col_of<L>(cb, s));
+}
+template <typename T, int R, int C, layout L>
+__device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, R, C, L>& src) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) *dst.at(row_of<L>(rb, s), col_of<L>(cb, s)) = src.data[rb][cb][s];
+    wave_fence();
+}
+template <typename T, int N, vlayout V>
+__device__ __forceinline__ void load(rv<T, N, V>& dst, const sv<T, N>& src) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b) {
+        if (V == vlayout::align) {
+            dst.data[b][0] = src.data[32 * b + lr()];
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[b][s] = src.data[col_of<layout::row>(b, s)];
+        }
+    }
+}
+template <typename T, int N, vlayout V>
+__device__ __forceinline__ void store(sv<T, N>& dst, const rv<T, N, V>& src) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b) {
+        if (V == vlayout::align) {
+            if (lg() == 0) dst.data[32 * b + lr()] = src.data[b][0];
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (lr() == 0) dst.data[col_of<layout::row>(b, s)] = src.data[b][s];
+        }
+    }
+    wave_fence();
+}
+
+// ---------------------------------------------------------------- products
+// D = A B + C on the 32x32x16 bf16 MFMA.  The product is issued transposed (the B fragment as
+// the MFMA's row operand) so that the accumulator comes out in ROW layout.
+namespace detail {
+template <typename TA, typename TB>
+__device__ __forceinline__ void mfma_block(float (&d)[16], const TA (&a)[16], const TB (&b)[16]) {
+    static_assert(sizeof(TA) == 2 && sizeof(TB) == 2, "products take bf16 operands");
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = d[e];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        bf16x8 fa, fb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { fa[e] = a[8 * h + e]; fb[e] = b[8 * h + e]; }
+        acc = mfma_32x32x16_bf16(fb, fa, acc);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) d[e] = acc[e];
+}
+}  // namespace detail
+
+#define TYR_TILE_MMA(NAME, ATYPE, BTYPE, KDIM, AIDX, BIDX)                                          \
+    template <int M, int N, int K>                                                                  \
+    __device__ __forceinline__ void NAME(rt<float, M, N, layout::row>& d, const ATYPE& a,           \
+                                         const BTYPE& b, const rt<float, M, N, layout::row>& c) {   \
+        _Pragma("unroll") for (int mb = 0; mb < M / 32; ++mb)                                       \
+        _Pragma("unroll") for (int nb = 0; nb < N / 32; ++nb) {                                     \
+            float acc[16];                                                                          \
+            _Pragma("unroll") for (int e = 0; e < 16; ++e) acc[e] = c.data[mb][nb][e];              \
+            _Pragma("unroll") for (int kb = 0; kb < KDIM / 32; ++kb)                                \
+                detail::mfma_block(acc, a.data AIDX, b.data BIDX);                                  \
+            _Pragma("unroll") for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[e];              \
+        }                                                                                           \
+    }
+#define TYR_TILE_COMMA ,
+// A[M,K] row, B[K,N] col
+TYR_TILE_MMA(mma_AB, rt<bf16 TYR_TILE_COMMA M TYR_TILE_COMMA K TYR_TILE_COMMA layout::row>,
+             rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA N TYR_TILE_COMMA layout::col>, K, [mb][kb], [kb][nb])
+// A[M,K] row, B[N,K] row
+TYR_TILE_MMA(mma_ABt, rt<bf16 TYR_TILE_COMMA M TYR_TILE_COMMA K TYR_TILE_COMMA layout::row>,
+             rt<bf16 TYR_TILE_COMMA N TYR_TILE_COMMA K TYR_TILE_COMMA layout::row>, K, [mb][kb], [nb][kb])
+// A[K,M] col, B[K,N] col
+TYR_TILE_MMA(mma_AtB, rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA M TYR_TILE_COMMA layout::col>,
+             rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA N TYR_TILE_COMMA layout::col>, K, [kb][mb], [kb][nb])
+// A[K,M] col, B[N,K] row
+TYR_TILE_MMA(mma_AtBt, rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA M TYR_TILE_COMMA layout::col>,
+             rt<bf16 TYR_TILE_COMMA N TYR_TILE_COMMA K TYR_TILE_COMMA layout::row>, K, [kb][mb], [nb][kb])
+#undef TYR_TILE_MMA
+
+// ---------------------------------------------------------------- element-wise
+// Arithmetic is done in f32 whatever the storage type; results are rounded to the storage type.
+template <typename OP, typename T, int R, int C, layout L>
+__device__ __forceinline__ void unary(rt<T, R, C, L>& dst, const rt<T, R, C, L>& src) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(OP::f(to_f(src.data[rb][cb][s])));
+}
+template <typename OP, typename T, int N, vlayout V>
+__device__ __forceinline__ void unary(rv<T, N, V>& dst, const rv<T, N, V>& src) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(OP::f(to_f(src.data[b][s])));
+}
+template <typename OP, typename T, int R, int C, layout L>
+__device__ __forceinline__ void binary(rt<T, R, C, L>& dst, const rt<T, R, C, L>& a, const rt<T, R, C, L>& b) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(OP::f(to_f(a.data[rb][cb][s]), to_f(b.data[rb][cb][s])));
+}
+template <typename OP, typename T, int N, vlayout V>
+__device__ __forceinline__ void binary(rv<T, N, V>& dst, const rv<T, N, V>& a, const rv<T, N, V>& b) {
+#pragma unroll
+    for (int bl = 0; bl < N / 32; ++bl)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s)
+            dst.data[bl][s] = from_f<T>(OP::f(to_f(a.data[bl][s]), to_f(b.data[bl][s])));
+}
+template <typename OP, typename T, int R, int C, layout L>
+__device__ __forceinline__ void scalar(rt<T, R, C, L>& dst, const rt<T, R, C, L>& src, float k) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(OP::f(to_f(src.data[rb][cb][s]), k));
+}
+template <typename OP, typename T, int N, vlayout V>
+__device__ __forceinline__ void scalar(rv<T, N, V>& dst, const rv<T, N, V>& src, float k) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(OP::f(to_f(src.data[b][s]), k));
+}
+// dst = a * b + c
+template <typename T, int R, int C, layout L>
+__device__ __forceinline__ void fma(rt<T, R, C, L>& dst, const rt<T, R, C, L>& a, const rt<T, R, C, L>& b,
+                                    const rt<T, R, C, L>& c) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT)
+        dst.data[rb][cb][s] = from_f<T>(fmaf(to_f(a.data[rb][cb][s]), to_f(b.data[rb][cb][s]), to_f(c.data[rb][cb][s])));
+}
+template <typename TD, typename TS, int R, int C, layout L>
+__device__ __forceinline__ void convert(rt<TD, R, C, L>& dst, const rt<TS, R, C, L>& src) {
+    typedef rt<TD, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<TD>(to_f(src.data[rb][cb][s]));
+}
+template <typename TD, typename TS, int N, vlayout V>
+__device__ __forceinline__ void convert(rv<TD, N, V>& dst, const rv<TS, N, V>& src) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<TD>(to_f(src.data[b][s]));
+}
+// The transpose of a ROW tile is the COL tile with the same registers (and back).
+template <typename T, int R, int C>
+__device__ __forceinline__ void transpose(rt<T, C, R, layout::col>& dst, const rt<T, R, C, layout::row>& src) {
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[cb][rb][s] = src.data[rb][cb][s];
+}
+template <typename T, int R, int C>
+__device__ __forceinline__ void transpose(rt<T, C, R, layout::row>& dst, const rt<T, R, C, layout::col>& src) {
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[cb][rb][s] = src.data[rb][cb][s];
+}
+// Same matrix, other layout: through an LDS tile the caller provides.
+template <typename T, int R, int C, layout LD, layout LS>
+__device__ __forceinline__ void swap_layout(rt<T, R, C, LD>& dst, const rt<T, R, C, LS>& src, st<T, R, C>& scratch) {
+    store(scratch, src);
+    load(dst, scratch);
+    wave_fence();
+}
+
+// column ranges at multiples of 32
+template <int START, typename T, int R, int C, int CS, layout L>
+__device__ __forceinline__ void slice_cols(rt<T, R, CS, L>& dst, const rt<T, R, C, L>& src) {
+    static_assert(START % 32 == 0 && START + CS <= C, "column slices start at multiples of 32");
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < CS / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[rb][cb][s] = src.data[rb][START / 32 + cb][s];
+}
+template <int START, typename T, int R, int C, int RS, layout L>
+__device__ __forceinline__ void slice_rows(rt<T, RS, C, L>& dst, const rt<T, R, C, L>& src) {
+    static_assert(START % 32 == 0 && START + RS <= R, "row slices start at multiples of 32");
+#pragma unroll
+    for (int rb = 0; rb < RS / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[rb][cb][s] = src.data[START / 32 + rb][cb][s];
+}
+template <typename T, int R, int CL, int CR, layout L>
+__device__ __forceinline__ void concat_cols(rt<T, R, CL + CR, L>& dst, const rt<T, R, CL, L>& left,
+                                            const rt<T, R, CR, L>& right) {
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) {
+#pragma unroll
+        for (int cb = 0; cb < CL / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[rb][cb][s] = left.data[rb][cb][s];
+#pragma unroll
+        for (int cb = 0; cb < CR / 32; ++cb)
+#pragma unroll
+            for (int s = 0; s < 16; ++s) dst.data[rb][CL / 32 + cb][s] = right.data[rb][cb][s];
+    }
+}
+
+// ---------------------------------------------------------------- masks
+template <typename KEEP, typename T, int R, int C, layout L>
+__device__ __forceinline__ void mask(rt<T, R, C, L>& dst, const rt<T, R, C, L>& src, float fill, int d = 0) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT)
+        dst.data[rb][cb][s] = KEEP::f(row_of<L>(rb, s), col_of<L>(cb, s), d) ? src.data[rb][cb][s] : from_f<T>(fill);
+}
+
+// ---------------------------------------------------------------- reductions and broadcasts (ROW tiles)
+// row_reduce: dst[i] = OP over j of src[i][j]  (ALIGN vector);  with `accum`: OP(that, accum[i]).
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void row_reduce(rv<T, R, vlayout::align>& dst, const rt<T, R, C, layout::row>& src) {
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) {
+        float acc = to_f(src.data[rb][0][0]);
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int s = (cb == 0 ? 1 : 0); s < 16; ++s) acc = OP::f(acc, to_f(src.data[rb][cb][s]));
+        dst.data[rb][0] = from_f<T>(OP::f(acc, xor32(acc)));
+    }
+}
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void row_reduce(rv<T, R, vlayout::align>& dst, const rt<T, R, C, layout::row>& src,
+                                           const rv<T, R, vlayout::align>& accum) {
+    rv<T, R, vlayout::align> tmp;
+    row_reduce<OP>(tmp, src);
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) dst.data[rb][0] = from_f<T>(OP::f(to_f(tmp.data[rb][0]), to_f(accum.data[rb][0])));
+}
+// col_reduce: dst[j] = OP over i of src[i][j]  (ORTHO vector)
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void col_reduce(rv<T, C, vlayout::ortho>& dst, const rt<T, R, C, layout::row>& src) {
+#pragma unroll
+    for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            float acc = to_f(src.data[0][cb][s]);
+#pragma unroll
+            for (int rb = 1; rb < R / 32; ++rb) acc = OP::f(acc, to_f(src.data[rb][cb][s]));
+#pragma unroll
+            for (int m = 1; m < 32; m <<= 1) acc = OP::f(acc, lane_xor(acc, m));
+            dst.data[cb][s] = from_f<T>(acc);
+        }
+}
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void col_reduce(rv<T, C, vlayout::ortho>& dst, const rt<T, R, C, layout::row>& src,
+                                           const rv<T, C, vlayout::ortho>& accum) {
+    rv<T, C, vlayout::ortho> tmp;
+    col_reduce<OP>(tmp, src);
+#pragma unroll
+    for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+        for (int s = 0; s < 16; ++s) dst.data[cb][s] = from_f<T>(OP::f(to_f(tmp.data[cb][s]), to_f(accum.data[cb][s])));
+}
+// dst[i][j] = OP(src[i][j], v[i])   (the DSL's *Col operations: v is a column vector)
+template <typename OP, typename T, typename TV, int R, int C>
+__device__ __forceinline__ void col_broadcast(rt<T, R, C, layout::row>& dst, const rt<T, R, C, layout::row>& src,
+                                              const rv<TV, R, vlayout::align>& v) {
+    typedef rt<T, R, C, layout::row> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(OP::f(to_f(src.data[rb][cb][s]), to_f(v.data[rb][0])));
+}
+// dst[i][j] = OP(src[i][j], v[j])   (the DSL's *Row operations: v is a row vector)
+template <typename OP, typename T, typename TV, int R, int C>
+__device__ __forceinline__ void row_broadcast(rt<T, R, C, layout::row>& dst, const rt<T, R, C, layout::row>& src,
+                                              const rv<TV, C, vlayout::ortho>& v) {
+    typedef rt<T, R, C, layout::row> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(OP::f(to_f(src.data[rb][cb][s]), to_f(v.data[cb][s])));
+}
+// dst[i][j] = v[i] / v[j]
+template <typename T, typename TV, int R, int C>
+__device__ __forceinline__ void broadcast_col(rt<T, R, C, layout::row>& dst, const rv<TV, R, vlayout::align>& v) {
+    typedef rt<T, R, C, layout::row> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(v.data[rb][0]));
+}
+template <typename T, typename TV, int R, int C>
+__device__ __forceinline__ void broadcast_row(rt<T, R, C, layout::row>& dst, const rv<TV, C, vlayout::ortho>& v) {
+    typedef rt<T, R, C, layout::row> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(v.data[cb][s]));
+}
+// dst[i][j] = a[i] * b[j]
+template <typename T, typename TV, int R, int C>
+__device__ __forceinline__ void outer(rt<T, R, C, layout::row>& dst, const rv<TV, R, vlayout::align>& a,
+                                      const rv<TV, C, vlayout::ortho>& b) {
+    typedef rt<T, R, C, layout::row> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(a.data[rb][0]) * to_f(b.data[cb][s]));
+}
+
+__device__ __forceinline__ void sync() { __syncthreads(); }
+
+}  // namespace wave
+}  // namespace tile
+}  // namespace tyr

@@ -1,0 +1,413 @@
+"""HIP emitter for the tile DSL: `Kernel` -> one gfx950 translation unit.
+
+The counterpart of the reference's CUDA emitter (Tyr/GPU/Codegen/EmitNew.lean:207-700 prints one
+ThunderKittens call per statement; Tyr/GPU/Codegen/Attribute.lean:318-386 prints the launcher).
+Here a statement becomes one call into the wave-level tile vocabulary of
+`tyr_amd/csrc/tile/tyr_tile.hpp`, and the launcher is a C-ABI function over raw pointers plus, for a
+build that has Lean and LibTorch headers, the `lean_launch_<kernel>` wrapper with the reference's
+signature and error strings.
+
+Statements that only exist for NVIDIA hardware paths (TMA, multimem, tcgen05, semaphores, named
+barriers, warp-group election) raise `UnsupportedStatement`; the asynchronous-MMA bookkeeping
+statements are no-ops because an MFMA is complete when its result is read.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+from .ir import GPU_FLOAT, K_SCALAR_TYPES, Kernel, Stmt, VarId, walk
+
+
+class UnsupportedStatement(NotImplementedError):
+    pass
+
+
+class LayoutConflict(ValueError):
+    pass
+
+
+CPP_TYPE = {"Float32": "float", "BFloat16": "bf16"}
+UNARY = {"Exp": "op_exp", "Exp2": "op_exp2", "Log": "op_log", "Log2": "op_log2", "Abs": "op_abs", "Relu": "op_relu",
+         "Copy": "op_copy", "Neg": "op_neg", "Sqrt": "op_sqrt", "Rsqrt": "op_rsqrt", "Tanh": "op_tanh",
+         "FastTanh": "op_tanh", "Sigmoid": "op_sigmoid", "Gelu": "op_gelu", "Silu": "op_silu", "Swish": "op_silu",
+         "Sin": "op_sin", "Cos": "op_cos", "Recip": "op_recip", "Square": "op_square", "Zero": "op_zero",
+         "One": "op_one", "PosInfty": "op_pos_infty", "NegInfty": "op_neg_infty"}
+BINARY = {"Add": "op_add", "Sub": "op_sub", "Mul": "op_mul", "Div": "op_div", "Max": "op_max", "Min": "op_min"}
+REDUCE = {"Max": "op_max", "Min": "op_min", "Sum": "op_add", "Prod": "op_mul"}
+MASK = {"MakeCausal": "keep_causal", "MakeCausalT": "keep_causal_t", "Tril": "keep_tril", "Triu": "keep_triu",
+        "RightFill": "keep_right_fill", "LeftFill": "keep_left_fill", "UpperFill": "keep_upper_fill",
+        "LowerFill": "keep_lower_fill"}
+NO_OPS = {"mmaFence", "mmaCommitGroup", "mmaAsyncWait", "fenceViewAsyncShared", "fenceProxyAsync"}
+NVIDIA_ONLY = {"declSemaphore", "loadAsync", "storeAsync", "storeAdd", "storeAddAsync", "storeMinAsync", "prefetch",
+               "tmaExpect", "tmaLoad", "tmaStore", "loadGlobalAsync", "storeGlobalAsync", "storeGlobalAdd",
+               "storeVecGlobalAdd", "storeVecGlobalAddCoord", "multimemLoadReduce", "multimemStore", "multimemRed",
+               "tcgen05Mma", "cpAsyncLoad", "tmaLoadAsync", "arrive", "arriveAndWait", "namedBarrierSync",
+               "namedBarrierArrive", "warpGroupIdx", "electOneSync", "semaphore", "ifWarpGroup", "cumsum", "cumprod",
+               "vecIota", "vecFillScalar"}
+
+
+def _cpp_type(dtype: str) -> str:
+    if dtype not in CPP_TYPE:
+        raise UnsupportedStatement(f"element type {dtype} has no gfx950 tile type yet (have {sorted(CPP_TYPE)})")
+    return CPP_TYPE[dtype]
+
+
+def _flt(x: float) -> str:
+    if x != x:
+        return "NAN"
+    if x in (float("inf"), float("-inf")):
+        return "INFINITY" if x > 0 else "-INFINITY"
+    return repr(float(x)) + "f"
+
+
+def infer_rv_layouts(kernel: Kernel) -> Dict[VarId, str]:
+    """align / ortho for every register vector (the reference infers naive / ortho / align the
+    same way, EmitNew.lean:100-200): what a vector is reduced from or broadcast along fixes its
+    layout, and element-wise vector statements tie their operands together."""
+    rvs = {s.v for s in walk(kernel.body) if s.op == "declRV"}
+    parent = {v: v for v in rvs}
+
+    def find(v):
+        while parent[v] != v:
+            parent[v] = parent[parent[v]]
+            v = parent[v]
+        return v
+
+    want: Dict[VarId, set] = {}
+
+    def need(v, lay):
+        if v in rvs:
+            want.setdefault(v, set()).add(lay)
+
+    def tie(*vs):
+        vs = [v for v in vs if v in rvs]
+        for v in vs[1:]:
+            parent[find(v)] = find(vs[0])
+
+    for s in walk(kernel.body):
+        if s.op == "reduce":
+            need(s.dst, "align" if s.axis == "Row" else "ortho")
+        elif s.op == "reduceAccum":
+            lay = "align" if s.axis == "Row" else "ortho"
+            need(s.dst, lay)
+            need(s.accum, lay)
+        elif s.op in ("broadcast", "binaryBroadcast"):
+            need(s.vec, "align" if s.axis == "Col" else "ortho")
+        elif s.op == "outer":
+            need(s.a, "align")
+            need(s.b, "ortho")
+        elif s.op in ("unary", "convert", "scalarMul", "scalarAdd"):
+            tie(s.dst, s.src)
+        elif s.op == "binary":
+            tie(s.dst, s.a, s.b)
+    groups: Dict[VarId, set] = {}
+    for v, lays in want.items():
+        groups.setdefault(find(v), set()).update(lays)
+    out = {}
+    for v in rvs:
+        lays = groups.get(find(v), set())
+        if len(lays) > 1:
+            raise LayoutConflict(f"RV layout conflict for {v.ident}")
+        out[v] = next(iter(lays)) if lays else "align"
+    return out
+
+
+class _Emitter:
+    def __init__(self, kernel: Kernel, max_waves: int = 4):
+        self.k = kernel
+        # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
+        # full 512-register file, and covers the 128-thread blocks the reference's runners launch
+        self.max_waves = max_waves
+        self.info: Dict[VarId, Stmt] = {}
+        for s in walk(kernel.body):
+            if s.op in ("declRT", "declST", "declRV", "declSV", "declGPtr", "declKVal"):
+                self.info[s.v] = s
+        self.rv_layout = infer_rv_layouts(kernel)
+
+    def kind(self, v: VarId) -> str:
+        s = self.info.get(v)
+        return s.op[4:] if s is not None else "scalar"
+
+    def is_vec(self, v):
+        return self.kind(v) in ("RV", "SV")
+
+    # ------------------------------------------------------------------ statements
+    def stmt(self, s: Stmt, ind: str) -> str:
+        op, I = s.op, (lambda v: v.ident)
+        if op in NVIDIA_ONLY:
+            raise UnsupportedStatement(f"{op} has no gfx950 lowering")
+        if op in NO_OPS:
+            return f"{ind}// {op}: nothing to do, an MFMA result is complete when it is read\n"
+        if op == "declRT":
+            return f"{ind}rt<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)};\n"
+        if op == "declST":
+            return f"{ind}__shared__ st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}> {I(s.v)};\n"
+        if op == "declRV":
+            return f"{ind}rv<{_cpp_type(s.dtype)}, {s.len}, vlayout::{self.rv_layout[s.v]}> {I(s.v)};\n"
+        if op == "declSV":
+            return f"{ind}__shared__ sv<{_cpp_type(s.dtype)}, {s.len}> {I(s.v)};\n"
+        if op == "declGPtr":
+            return f"{ind}// param: {_cpp_type(s.dtype)}* {s.name} ({I(s.v)})\n"
+        if op == "declKVal":
+            return f"{ind}// param: {s.name} ({I(s.v)})\n"
+        if op in ("load", "store"):
+            return f"{ind}wave::{op}({I(s.dst)}, {I(s.src)});\n"
+        if op in ("loadGlobal", "storeGlobal"):
+            tile = self.info[s.dst if op == "loadGlobal" else s.src]
+            at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)} * {tile.rows}, (int){I(s.coordC)} * {tile.cols}}}"
+            return f"{ind}wave::{'load' if op == 'loadGlobal' else 'store'}({I(s.dst)}, {I(s.src)}, {at});\n"
+        if op in ("loadVecGlobal", "storeVecGlobal"):
+            return f"{ind}wave::{'load' if op == 'loadVecGlobal' else 'store'}({I(s.dst)}, {I(s.src)}, (int){I(s.offset)});\n"
+        if op in ("loadVecGlobalCoord", "storeVecGlobalCoord"):
+            at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)}, (int){I(s.coordC)}}}"
+            return f"{ind}wave::{'load' if op == 'loadVecGlobalCoord' else 'store'}({I(s.dst)}, {I(s.src)}, {at});\n"
+        if op == "loadScalarGlobal":
+            return f"{ind}const auto {I(s.dst)} = {I(s.src)}.ptr[{I(s.offset)}];\n"
+        if op == "storeScalarGlobal":
+            return f"{ind}{I(s.dst)}.ptr[{I(s.offset)}] = {I(s.src)};\n"
+        if op == "layoutDim":
+            return f"{ind}const int {I(s.dst)} = {I(s.src)}.{s.axis.lower()}();\n"
+        if op == "mma":
+            return f"{ind}wave::mma_{s.trans}({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.c)});\n"
+        if op == "mm":
+            return (f"{ind}wave::unary<op_zero>({I(s.dst)}, {I(s.dst)});\n"
+                    f"{ind}wave::mma_{s.trans}({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.dst)});\n")
+        if op == "unary":
+            return f"{ind}wave::unary<{UNARY[s.args[0]]}>({I(s.dst)}, {I(s.src)});\n"
+        if op == "binary":
+            return f"{ind}wave::binary<{BINARY[s.args[0]]}>({I(s.dst)}, {I(s.a)}, {I(s.b)});\n"
+        if op == "ternary":
+            if s.args[0] != "FMA":
+                raise UnsupportedStatement(f"ternary {s.args[0]} has no gfx950 lowering")
+            return f"{ind}wave::fma({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.c)});\n"
+        if op in ("scalarMul", "scalarAdd"):
+            f = "op_mul" if op == "scalarMul" else "op_add"
+            return f"{ind}wave::scalar<{f}>({I(s.dst)}, {I(s.src)}, {_flt(s.scalar)});\n"
+        if op == "broadcast":
+            return f"{ind}wave::broadcast_{s.axis.lower()}({I(s.dst)}, {I(s.vec)});\n"
+        if op == "binaryBroadcast":
+            return f"{ind}wave::{s.axis.lower()}_broadcast<{BINARY[s.args[0]]}>({I(s.dst)}, {I(s.tile)}, {I(s.vec)});\n"
+        if op in ("reduce", "reduceAccum"):
+            if s.axis == "Full":
+                raise UnsupportedStatement("full reductions have no gfx950 lowering yet")
+            tail = f", {I(s.accum)}" if op == "reduceAccum" else ""
+            return f"{ind}wave::{s.axis.lower()}_reduce<{REDUCE[s.args[0]]}>({I(s.dst)}, {I(s.src)}{tail});\n"
+        if op == "outer":
+            return f"{ind}wave::outer({I(s.dst)}, {I(s.a)}, {I(s.b)});\n"
+        if op == "transpose":
+            if s.dst == s.src:
+                raise UnsupportedStatement("in-place transpose changes the tile's type; use a second tile")
+            return f"{ind}wave::transpose({I(s.dst)}, {I(s.src)});\n"
+        if op == "swapLayout":
+            t = self.info[s.src]
+            return (f"{ind}{{\n{ind}  __shared__ st<{_cpp_type(t.dtype)}, {t.rows}, {t.cols}> {I(s.dst)}_swap;\n"
+                    f"{ind}  wave::swap_layout({I(s.dst)}, {I(s.src)}, {I(s.dst)}_swap);\n{ind}}}\n")
+        if op == "convert":
+            return f"{ind}wave::convert({I(s.dst)}, {I(s.src)});\n"
+        if op == "mask":
+            tag = s.args[0]
+            if tag[0] not in MASK:
+                raise UnsupportedStatement(f"mask {tag[0]} has no gfx950 lowering yet")
+            fill = _flt(0.0 if s.fillVal is None else s.fillVal)
+            d = f", {tag[1]}" if len(tag) > 1 else ""
+            return f"{ind}wave::mask<{MASK[tag[0]]}>({I(s.dst)}, {I(s.src)}, {fill}{d});\n"
+        if op == "sliceRows":
+            return f"{ind}wave::slice_rows<{s.startRow}>({I(s.dst)}, {I(s.src)});\n"
+        if op == "sliceCols":
+            return f"{ind}wave::slice_cols<{s.startCol}>({I(s.dst)}, {I(s.src)});\n"
+        if op == "concatCols":
+            return f"{ind}wave::concat_cols({I(s.dst)}, {I(s.left)}, {I(s.right)});\n"
+        if op == "sync":
+            return f"{ind}wave::sync();\n"
+        if op == "forLoop":
+            return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < {s.hi}; ++{I(s.v)}) {{\n" + self.body(s.body, ind + "  ") +
+                    f"{ind}}}\n")
+        if op == "forLoopVal":
+            return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < (int){I(s.hi)}; ++{I(s.v)}) {{\n" +
+                    self.body(s.body, ind + "  ") + f"{ind}}}\n")
+        if op == "ifStmt":
+            out = f"{ind}if ({I(s.cond)}) {{\n" + self.body(s.thenBody, ind + "  ") + f"{ind}}}"
+            if s.elseBody:
+                out += " else {\n" + self.body(s.elseBody, ind + "  ") + f"{ind}}}"
+            return out + "\n"
+        if op == "comment":
+            return f"{ind}// {s.text}\n"
+        if op == "getBlockIdx":
+            return f"{ind}const int {I(s.dst)} = blockIdx.{'xyz'[s.axis]};\n"
+        if op == "getThreadIdx":
+            return f"{ind}const int {I(s.dst)} = threadIdx.{'xyz'[s.axis]};\n"
+        if op == "constInt":
+            return f"{ind}const int {I(s.dst)} = {s.value};\n"
+        if op == "constFloat":
+            return f"{ind}const float {I(s.dst)} = {_flt(s.value)};\n"
+        if op == "scalarUnary":
+            e = f"-{I(s.src)}" if s.args[0] == "Neg" else f"__expf((float){I(s.src)})"
+            return f"{ind}const auto {I(s.dst)} = {e};\n"
+        if op == "scalarCompare":
+            c = {"Eq": "==", "Lt": "<", "Le": "<=", "Gt": ">", "Ge": ">="}[s.args[0]]
+            return f"{ind}const bool {I(s.dst)} = {I(s.a)} {c} {I(s.b)};\n"
+        if op == "scalarBinary":
+            o = s.args[0]
+            if o in ("Min", "Max"):
+                e = f"({I(s.a)} {'<' if o == 'Min' else '>'} {I(s.b)} ? {I(s.a)} : {I(s.b)})"
+            else:
+                sym = {"Add": "+", "Sub": "-", "Mul": "*", "Div": "/", "Mod": "%"}[o]
+                e = f"{I(s.a)} {sym} {I(s.b)}"
+            return f"{ind}const auto {I(s.dst)} = {e};\n"
+        if op == "scalarSelect":
+            return f"{ind}const auto {I(s.dst)} = {I(s.cond)} ? {I(s.ifTrue)} : {I(s.ifFalse)};\n"
+        if op == "raw":
+            return f"{ind}{s.code}\n"
+        raise UnsupportedStatement(op)
+
+    def body(self, stmts, ind: str) -> str:
+        return "".join(self.stmt(s, ind) for s in stmts)
+
+    # ------------------------------------------------------------------ kernel + launchers
+    def param_decls(self):
+        """(kernel parameter text, VarId) in signature order: the k-th parameter is the k-th
+        declGPtr / declKVal statement."""
+        decls = [s for s in self.k.body if s.op in ("declGPtr", "declKVal")]
+        assert len(decls) == len(self.k.params), "every parameter needs its declGPtr / declKVal statement"
+        out = []
+        for p, d in zip(self.k.params, decls):
+            if p.isPointer:
+                out.append((f"gl<{_cpp_type(p.dtype)}> {d.v.ident}", d.v, p))
+            else:
+                out.append((f"{K_SCALAR_TYPES[p.scalarTy]} {d.v.ident}", d.v, p))
+        return out
+
+    def kernel_text(self) -> str:
+        sig = ", ".join(t for t, _, _ in self.param_decls())
+        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" +
+                self.body(self.k.body, "  ") + "}\n")
+
+    def launcher_signature(self) -> str:
+        cparams = []
+        for _, _, p in self.param_decls():
+            if p.isPointer:
+                cparams += [f"void* {p.name}", f"const int64_t* {p.name}_shape", f"int {p.name}_ndim"]
+            else:
+                cparams.append(f"{K_SCALAR_TYPES[p.scalarTy]} {p.name}")
+        cparams += ["uint64_t grid_x", "uint64_t grid_y", "uint64_t grid_z", "uint64_t block_x", "uint64_t block_y",
+                    "uint64_t block_z", "uint64_t shared_mem", "void* stream"]
+        return f"int tyr_launch_{self.k.name}({', '.join(cparams)})"
+
+    def launcher_text(self) -> str:
+        name, decls = self.k.name, self.param_decls()
+        cparams, setup, args = [], [], []
+        for i, (_, v, p) in enumerate(decls):
+            if p.isPointer:
+                cparams += [f"void* {p.name}", f"const int64_t* {p.name}_shape", f"int {p.name}_ndim"]
+                setup.append(
+                    f"  if ({p.name} == nullptr || {p.name}_ndim < 0 || {p.name}_ndim > 4) return -2;\n"
+                    f"  int s{i}[4] = {{1, 1, 1, 1}};\n"
+                    f"  for (int i = 0; i < {p.name}_ndim; ++i) s{i}[4 - {p.name}_ndim + i] = (int){p.name}_shape[i];\n"
+                    f"  gl<{_cpp_type(p.dtype)}> g{i}{{static_cast<{_cpp_type(p.dtype)}*>({p.name}), s{i}[0], s{i}[1], s{i}[2], s{i}[3]}};\n")
+                args.append(f"g{i}")
+            else:
+                cparams.append(f"{K_SCALAR_TYPES[p.scalarTy]} {p.name}")
+                args.append(p.name)
+        cparams += ["uint64_t grid_x", "uint64_t grid_y", "uint64_t grid_z", "uint64_t block_x", "uint64_t block_y",
+                    "uint64_t block_z", "uint64_t shared_mem", "void* stream"]
+        return (
+            f"// C ABI: tensors as (device pointer, shape, rank <= 4), then the kernel's scalars, then the launch\n"
+            f"// geometry of the reference launcher (Tyr/GPU/Codegen/Attribute.lean:344-386).  A 32-thread warp of\n"
+            f"// the requested block becomes one 64-lane wave.  Returns 0, -2 (bad argument) or -1 (launch error).\n"
+            f"extern \"C\" int tyr_launch_{name}({', '.join(cparams)}) {{\n" + "".join(setup) +
+            f"  const uint64_t threads = block_x * block_y * block_z;\n"
+            f"  if (threads == 0 || grid_x * grid_y * grid_z == 0) return -2;\n"
+            f"  const unsigned waves = (unsigned)((threads + 31) / 32);\n"
+            f"  if (waves > {self.max_waves}) return -2;\n"
+            f"  hipLaunchKernelGGL({name}, dim3((unsigned)grid_x, (unsigned)grid_y, (unsigned)grid_z), dim3(64 * waves), "
+            f"(size_t)shared_mem, static_cast<hipStream_t>(stream), {', '.join(args)});\n"
+            f"  return hipGetLastError() == hipSuccess ? 0 : -1;\n}}\n")
+
+    def lean_launcher_text(self) -> str:
+        """`lean_launch_<kernel>` with the reference's signature, checks and messages
+        (Attribute.lean:318-386), over the C-ABI launcher above."""
+        name, decls = self.k.name, self.param_decls()
+        lparams, setup, args = [], [], []
+        for i, (_, v, p) in enumerate(decls):
+            if p.isPointer:
+                lparams.append(f"b_lean_obj_arg {p.name}")
+                setup.append(
+                    f"  auto t{i} = borrowTensor({p.name});\n"
+                    f"  if (!t{i}.is_cuda()) return tyr_dsl_io_error(\"{p.name} must be a CUDA tensor\");\n"
+                    f"  if (!t{i}.is_contiguous()) return tyr_dsl_io_error(\"{p.name} must be contiguous\");\n"
+                    f"  if (t{i}.dim() > 4) return tyr_dsl_io_error(\"{p.name} must have dim <= 4\");\n"
+                    f"  int64_t shape{i}[4] = {{1, 1, 1, 1}};\n"
+                    f"  for (int i = 0; i < (int)t{i}.dim(); ++i) shape{i}[i] = t{i}.size(i);\n")
+                args += [f"t{i}.data_ptr()", f"shape{i}", f"(int)t{i}.dim()"]
+            else:
+                lparams.append(f"{K_SCALAR_TYPES[p.scalarTy]} {p.name}")
+                args.append(p.name)
+        lparams += ["uint64_t grid_x", "uint64_t grid_y", "uint64_t grid_z", "uint64_t block_x", "uint64_t block_y",
+                    "uint64_t block_z", "uint64_t shared_mem", "uint64_t stream", "lean_object* /* world */"]
+        args += ["grid_x", "grid_y", "grid_z", "block_x", "block_y", "block_z", "shared_mem",
+                 "reinterpret_cast<void*>(stream)"]
+        return (f"extern \"C\" lean_object* lean_launch_{name}({', '.join(lparams)}) {{\n  try {{\n" +
+                "".join("  " + l + "\n" for l in "".join(setup).splitlines()) +
+                f"    const int rc = tyr_launch_{name}({', '.join(args)});\n"
+                f"    if (rc == -2) return tyr_dsl_io_error(\"invalid launch arguments for {name}\");\n"
+                f"    if (rc != 0) return tyr_dsl_io_error(hipGetErrorString(hipGetLastError()));\n"
+                f"    return lean_io_result_mk_ok(lean_box(0));\n"
+                f"  }} catch (const std::exception& e) {{\n    return tyr_dsl_io_error(e.what());\n  }}\n}}\n")
+
+
+PREAMBLE = """// Emitted from the tile DSL for gfx950; do not edit.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "tile/tyr_tile.hpp"
+
+using namespace tyr::tile;
+
+"""
+
+LEAN_PREAMBLE = """#if defined(__has_include)
+#if __has_include(<lean/lean.h>) && __has_include(<torch/torch.h>)
+#define TYR_HAVE_LEAN 1
+#endif
+#endif
+#ifdef TYR_HAVE_LEAN
+#include <lean/lean.h>
+#include <torch/torch.h>
+torch::Tensor borrowTensor(b_lean_obj_arg o);   // cc/src/tyr.cpp:127-148
+static lean_object* tyr_dsl_io_error(const char* msg) {
+  return lean_io_result_mk_error(lean_mk_io_user_error(lean_mk_string(msg)));
+}
+"""
+
+
+def emit_header(kernels: List[Kernel], cites: Dict[str, str]) -> str:
+    """C declarations of the launchers of `kernels`; `cites` maps a kernel name to the reference
+    definition whose generated `lean_launch_<kernel>` (Attribute.lean:344-386) the entry point stands in for."""
+    out = ("/* C ABI of the tile programs emitted for gfx950 (libtyr_dsl.so).  Generated by tyr_amd.dsl; do not edit.\n"
+           " *\n"
+           " * Every entry point replaces the launcher the reference generates for the same kernel,\n"
+           " * `lean_launch_<kernel>` (Tyr/GPU/Codegen/Attribute.lean:344-386): tensors arrive as (device pointer,\n"
+           " * shape, rank <= 4; right-aligned into batch, depth, rows, cols as the reference does,\n"
+           " * Attribute.lean:337-342), then the kernel's scalar parameters, then grid, block, dynamic shared\n"
+           " * memory and the stream.  A 32-thread warp of the requested block is run as one 64-lane wave.\n"
+           " * Returns 0 on success, -2 for an invalid argument, -1 if the launch failed. */\n"
+           "#ifndef TYR_DSL_KERNELS_H\n#define TYR_DSL_KERNELS_H\n\n#include <stdint.h>\n\n"
+           "#ifdef __cplusplus\nextern \"C\" {\n#endif\n\n")
+    for k in kernels:
+        out += f"/* {cites[k.name]} */\n{_Emitter(k).launcher_signature()};\n\n"
+    return out + "#ifdef __cplusplus\n}\n#endif\n\n#endif /* TYR_DSL_KERNELS_H */\n"
+
+
+def emit_kernel(kernel: Kernel) -> str:
+    """Device code of one kernel (no includes)."""
+    return _Emitter(kernel).kernel_text()
+
+
+def emit_translation_unit(kernels: List[Kernel]) -> str:
+    """One .hip file: every kernel, its C-ABI launcher, and (where Lean headers exist) its
+    `lean_launch_*` wrapper."""
+    ems = [_Emitter(k) for k in kernels]
+    out = PREAMBLE
+    for e in ems:
+        out += e.kernel_text() + "\n" + e.launcher_text() + "\n"
+    out += LEAN_PREAMBLE + "".join(e.lean_launcher_text() + "\n" for e in ems) + "#endif  // TYR_HAVE_LEAN\n"
+    return out

@@ -1,0 +1,298 @@
+"""The reference's end-to-end tested tile programs, written against `KernelBuilder`.
+
+Each function builds the same statement sequence as the Lean definition it cites; together they
+are the kernels the reference ships runners for (Examples/GPU/Run{Copy,Rotary,LayerNorm,FlashAttn}.lean)
+plus its canonical GEMM example.
+"""
+from __future__ import annotations
+
+from .builder import KernelBuilder
+from .ir import Kernel
+
+
+def copy64x64() -> Kernel:
+    """Tyr/GPU/Kernels/Copy.lean:16-26 -- one 64x64 f32 tile, global -> LDS -> registers and back."""
+    k = KernelBuilder("copy64x64")
+    inp = k.gptr("Float32", "input")
+    out = k.gptr("Float32", "output")
+    k.comment("ThunderKittens-style minimal copy kernel")
+    coord = k.blockCoord2D()
+    reg = k.allocRT("Float32", 64, 64)
+    smem = k.allocST("Float32", 64, 64)
+    k.loadGlobal(smem, inp, coord)
+    k.load(reg, smem)
+    k.store(smem, reg)
+    k.storeGlobal(out, smem, coord)
+    k.sync()
+    return k.build()
+
+
+def rotaryFwd() -> Kernel:
+    """Tyr/GPU/Kernels/Rotary.lean:13-62 -- RoPE on one 64x64 tile split as [x1 | x2]."""
+    k = KernelBuilder("rotaryFwd")
+    x_ptr = k.gptr("Float32", "x_ptr")
+    sin_ptr = k.gptr("Float32", "sin_ptr")
+    cos_ptr = k.gptr("Float32", "cos_ptr")
+    out_ptr = k.gptr("Float32", "out_ptr")
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    coord = k.blockCoord2D()
+
+    x = k.allocRT("Float32", 64, 64)
+    x1 = k.allocRT("Float32", 64, 32)
+    x2 = k.allocRT("Float32", 64, 32)
+    sinT = k.allocRT("Float32", 64, 32)
+    cosT = k.allocRT("Float32", 64, 32)
+    y1 = k.allocRT("Float32", 64, 32)
+    y2 = k.allocRT("Float32", 64, 32)
+    tmp = k.allocRT("Float32", 64, 32)
+    negX2 = k.allocRT("Float32", 64, 32)
+    out = k.allocRT("Float32", 64, 64)
+
+    xShared = k.allocST("Float32", 64, 64)
+    sinShared = k.allocST("Float32", 64, 32)
+    cosShared = k.allocST("Float32", 64, 32)
+    outShared = k.allocST("Float32", 64, 64)
+
+    k.loadGlobal(xShared, x_ptr, coord)
+    k.loadGlobal(sinShared, sin_ptr, coord)
+    k.loadGlobal(cosShared, cos_ptr, coord)
+    k.sync()
+
+    k.load(x, xShared)
+    k.load(sinT, sinShared)
+    k.load(cosT, cosShared)
+
+    k.sliceCols(x1, x, 0, 32)
+    k.sliceCols(x2, x, 32, 32)
+
+    # y1 = x1*cos - x2*sin
+    k.mul(y1, x1, cosT)
+    k.neg(negX2, x2)
+    k.mul(negX2, negX2, sinT)
+    k.add(y1, y1, negX2)
+
+    # y2 = x2*cos + x1*sin
+    k.mul(y2, x2, cosT)
+    k.mul(tmp, x1, sinT)
+    k.add(y2, y2, tmp)
+
+    k.concatCols(out, y1, y2)
+
+    k.store(outShared, out)
+    k.sync()
+    k.storeGlobal(out_ptr, outShared, coord)
+    return k.build()
+
+
+def tkFusedLayerNormResidual1024() -> Kernel:
+    """Tyr/GPU/Kernels/FusedLayerNorm.lean:28-126 -- residual add + LayerNorm over d_model = 1024 on
+    64-row blocks, two passes over sixteen 64x64 tiles."""
+    k = KernelBuilder("tkFusedLayerNormResidual1024")
+    x_ptr = k.gptr("BFloat16", "x_ptr")
+    residual_ptr = k.gptr("BFloat16", "residual_ptr")
+    weight_ptr = k.gptr("BFloat16", "weight_ptr")
+    bias_ptr = k.gptr("BFloat16", "bias_ptr")
+    out_ptr = k.gptr("BFloat16", "out_ptr")
+    out_resid_ptr = k.gptr("BFloat16", "out_resid_ptr")
+    k.comment("ThunderKittens-style layernorm + residual on 64x1024 tiles")
+
+    hiddenTiles = 16
+    invHidden = 0.0009765625
+    eps = 1.0e-5
+
+    coord = k.blockCoord2D()
+
+    x = k.allocRT("BFloat16", 64, 64)
+    residual = k.allocRT("BFloat16", 64, 64)
+    outResid = k.allocRT("BFloat16", 64, 64)
+    outResidF = k.allocRT("Float32", 64, 64)
+    centered = k.allocRT("Float32", 64, 64)
+    sq = k.allocRT("Float32", 64, 64)
+
+    tileShared = k.allocST("BFloat16", 64, 64)
+
+    sum_ = k.zeroRV("Float32", 64)
+    sumSq = k.zeroRV("Float32", 64)
+    tmpSum = k.allocRV("Float32", 64)
+    tmpSqSum = k.allocRV("Float32", 64)
+    mean = k.allocRV("Float32", 64)
+    meanSq = k.allocRV("Float32", 64)
+    var = k.allocRV("Float32", 64)
+    invStd = k.allocRV("Float32", 64)
+
+    weightShared = k.allocSV("BFloat16", 64)
+    biasShared = k.allocSV("BFloat16", 64)
+    weightRV = k.allocRV("BFloat16", 64)
+    biasRV = k.allocRV("BFloat16", 64)
+    weightF = k.allocRV("Float32", 64)
+    biasF = k.allocRV("Float32", 64)
+
+    k.comment("Pass 1: out_resid and row statistics across full hidden dimension")
+    with k.krange(0, hiddenTiles) as hiddenIdx:
+        tileCoord = coord.withCol(hiddenIdx.id)
+
+        k.loadGlobal(tileShared, x_ptr, tileCoord)
+        k.sync()
+        k.load(x, tileShared)
+
+        k.loadGlobal(tileShared, residual_ptr, tileCoord)
+        k.sync()
+        k.load(residual, tileShared)
+
+        k.add(outResid, x, residual)
+        k.store(tileShared, outResid)
+        k.sync()
+        k.storeGlobal(out_resid_ptr, tileShared, tileCoord)
+
+        k.convert(outResidF, outResid)
+        k.rowSum(tmpSum, outResidF)
+        k.addVec(sum_, sum_, tmpSum)
+        k.mul(sq, outResidF, outResidF)
+        k.rowSum(tmpSqSum, sq)
+        k.addVec(sumSq, sumSq, tmpSqSum)
+
+    k.scalarMulVec(mean, sum_, invHidden)
+    k.scalarMulVec(var, sumSq, invHidden)
+    k.mulVec(meanSq, mean, mean)
+    k.subVec(var, var, meanSq)
+    k.scalarAddVec(var, var, eps)
+    k.rsqrtVec(invStd, var)
+
+    k.comment("Pass 2: normalize + affine (weight, bias)")
+    with k.krange(0, hiddenTiles) as hiddenIdx:
+        tileCoord = coord.withCol(hiddenIdx.id)
+
+        k.loadGlobal(tileShared, out_resid_ptr, tileCoord)
+        k.sync()
+        k.load(outResid, tileShared)
+        k.convert(outResidF, outResid)
+
+        k.loadVecGlobalCol(weightShared, weight_ptr, tileCoord)
+        k.loadVec(weightRV, weightShared)
+        k.convertVec(weightF, weightRV)
+
+        k.loadVecGlobalCol(biasShared, bias_ptr, tileCoord)
+        k.loadVec(biasRV, biasShared)
+        k.convertVec(biasF, biasRV)
+
+        k.subCol(centered, outResidF, mean)
+        k.mulCol(centered, centered, invStd)
+        k.mulRow(centered, centered, weightF)
+        k.addRow(centered, centered, biasF)
+
+        k.convert(outResid, centered)
+        k.store(tileShared, outResid)
+        k.sync()
+        k.storeGlobal(out_ptr, tileShared, tileCoord)
+    return k.build()
+
+
+def simpleGemm(numKBlocks: int = 8) -> Kernel:
+    """Tyr/GPU/Kernels/Examples.lean:23-65 -- C[64x64 tile] = sum over numKBlocks of A tile x B tile,
+    bf16 operands, f32 accumulator and output."""
+    k = KernelBuilder("simpleGemm")
+    aPtr = k.gptr("BFloat16", "aPtr")
+    bPtr = k.gptr("BFloat16", "bPtr")
+    cPtr = k.gptr("Float32", "cPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    k.comment("=== Example GEMM ===")
+    coord = k.blockCoord2D()
+
+    a = k.allocRT("BFloat16", 64, 64)
+    b = k.allocRT("BFloat16", 64, 64, "Col")
+    c = k.zeroRT("Float32", 64, 64)
+
+    aS = k.allocST("BFloat16", 64, 64)
+    bS = k.allocST("BFloat16", 64, 64, "Col")
+    cS = k.allocST("Float32", 64, 64)
+
+    with k.krange(0, numKBlocks) as kBlk:
+        k.loadGlobal(aS, aPtr, coord.withCol(kBlk.id))
+        k.loadGlobal(bS, bPtr, coord.withRow(kBlk.id))
+        k.sync()
+        k.load(a, aS)
+        k.load(b, bS)
+        k.mma(c, a, b, c)
+        k.sync()
+
+    k.store(cS, c)
+    k.storeGlobal(cPtr, cS, coord)
+    return k.build()
+
+
+def tkFlashAttnFwd2BlockLse() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:71-128 -- attention forward of one 64-row query tile over two
+    64-row KV blocks (D = 64, scale 1/8), O in bf16 and LSE = ln(l) + m in f32."""
+    k = KernelBuilder("tkFlashAttnFwd2BlockLse")
+    q_ptr = k.gptr("BFloat16", "q_ptr")
+    k_ptr = k.gptr("BFloat16", "k_ptr")
+    v_ptr = k.gptr("BFloat16", "v_ptr")
+    o_ptr = k.gptr("BFloat16", "o_ptr")
+    lse_ptr = k.gptr("Float32", "lse_ptr")
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    tileSize = 64
+    numKvBlocks = 2
+    scale = 0.125
+
+    coord = k.blockCoord2D()
+
+    q = k.allocRT("BFloat16", tileSize, tileSize)
+    kt = k.allocRT("BFloat16", tileSize, tileSize)
+    v = k.allocRT("BFloat16", tileSize, tileSize, "Col")
+    o = k.zeroRT("Float32", tileSize, tileSize)
+
+    softmaxState = k.allocSoftmaxState("Float32", tileSize)
+
+    qShared = k.allocST("BFloat16", tileSize, tileSize)
+    kShared = k.allocST("BFloat16", tileSize, tileSize)
+    vShared = k.allocST("BFloat16", tileSize, tileSize, "Col")
+    oShared = k.allocST("BFloat16", tileSize, tileSize)
+    lseShared = k.allocSV("Float32", tileSize)
+
+    k.loadGlobal(qShared, q_ptr, coord)
+    k.sync()
+    k.load(q, qShared)
+
+    with k.krange(0, numKvBlocks) as kvIdx:
+        s = k.zeroRT("Float32", tileSize, tileSize)
+        p = k.allocRT("BFloat16", tileSize, tileSize)
+
+        k.loadGlobal(kShared, k_ptr, coord.withRow(kvIdx.id))
+        k.loadGlobal(vShared, v_ptr, coord.withRow(kvIdx.id))
+        k.sync()
+        k.load(kt, kShared)
+        k.load(v, vShared)
+
+        k.mmaT(s, q, kt, s)
+        k.scalarMul(s, s, scale)
+        k.onlineSoftmax(s, o, softmaxState)
+        k.convert(p, s)
+        k.mma(o, p, v, o)
+        k.sync()
+
+    k.finalizeSoftmax(o, softmaxState)
+    lse = k.computeLSE(softmaxState)
+
+    oBf16 = k.allocRT("BFloat16", tileSize, tileSize)
+    k.convert(oBf16, o)
+    k.store(oShared, oBf16)
+    k.storeGlobal(o_ptr, oShared, coord)
+
+    k.storeVec(lseShared, lse)
+    k.storeVecGlobalRow(lse_ptr, lseShared, coord)
+    return k.build()
+
+
+# kernel name -> the reference definition it restates
+CITES = {
+    "copy64x64": "Tyr/GPU/Kernels/Copy.lean:16-26 (runner Examples/GPU/RunCopy.lean:28)",
+    "rotaryFwd": "Tyr/GPU/Kernels/Rotary.lean:13-62 (runner Examples/GPU/RunRotary.lean:63)",
+    "tkFusedLayerNormResidual1024": "Tyr/GPU/Kernels/FusedLayerNorm.lean:28-126 (runner Examples/GPU/RunLayerNorm.lean:67)",
+    "simpleGemm": "Tyr/GPU/Kernels/Examples.lean:23-65",
+    "tkFlashAttnFwd2BlockLse": "Tyr/GPU/Kernels/MhaH100.lean:71-128 (runner Examples/GPU/RunFlashAttn.lean:81)",
+}
+ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, tkFlashAttnFwd2BlockLse)
