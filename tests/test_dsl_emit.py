@@ -179,3 +179,19 @@ def test_launcher_validates_on_the_host():
     assert fn(p, shape, 4, p, shape, 4, 0, 1, 1, 128, 1, 1, 0, None) == -2             # empty grid
     assert fn(p, shape, 4, p, shape, 4, 1, 1, 1, 0, 1, 1, 0, None) == -2               # empty block
     assert fn(p, shape, 4, p, shape, 4, 1, 1, 1, 256, 1, 1, 0, None) == -2             # more warps than compiled for
+
+
+def test_statement_coverage_programs_lower_and_are_built():
+    # every statement kind the emitter lowers appears in some program that runs on the GPU tests
+    from tyr_amd.dsl import op_programs, runtime
+    from tyr_amd.dsl.emit import NO_OPS, NVIDIA_ONLY
+    used = set()
+    for f in kernels.ALL + op_programs.ALL:
+        k = f()
+        dsl.emit_kernel(k)
+        used |= {s.op for s in walk(k.body)}
+    lowered = set(KSTMT_FIELDS) - NVIDIA_ONLY - NO_OPS
+    assert lowered - used == set(), lowered - used
+    L = runtime.load_op_programs()
+    for f in op_programs.ALL:
+        assert hasattr(L, f"tyr_launch_{f().name}")

@@ -438,6 +438,31 @@ __device__ __forceinline__ void mask(rt<T, R, C, L>& dst, const rt<T, R, C, L>& 
     TYR_TILE_FOR_BLOCKS(RT)
         dst.data[rb][cb][s] = KEEP::f(row_of<L>(rb, s), col_of<L>(cb, s), d) ? src.data[rb][cb][s] : from_f<T>(fill);
 }
+// rows < r0 of columns >= c0 take `fill`
+template <typename T, int R, int C, layout L>
+__device__ __forceinline__ void mask_upper_right(rt<T, R, C, L>& dst, const rt<T, R, C, L>& src, float fill, int r0, int c0) {
+    typedef rt<T, R, C, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT)
+        dst.data[rb][cb][s] = (row_of<L>(rb, s) < r0 && col_of<L>(cb, s) >= c0) ? from_f<T>(fill) : src.data[rb][cb][s];
+}
+// v[i] = start + step * i ;  v[i] = x
+template <typename T, int N, vlayout V>
+__device__ __forceinline__ void iota(rv<T, N, V>& dst, float start, float step) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s) {
+            const int i = V == vlayout::align ? 32 * b + lr() : col_of<layout::row>(b, s);
+            dst.data[b][s] = from_f<T>(start + step * (float)i);
+        }
+}
+template <typename T, int N, vlayout V>
+__device__ __forceinline__ void fill(rv<T, N, V>& dst, float x) {
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(x);
+}
 
 // ---------------------------------------------------------------- reductions and broadcasts (ROW tiles)
 // row_reduce: dst[i] = OP over j of src[i][j]  (ALIGN vector);  with `accum`: OP(that, accum[i]).

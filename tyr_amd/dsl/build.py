@@ -6,7 +6,7 @@ from __future__ import annotations
 import os
 import subprocess
 
-from . import kernels
+from . import kernels, op_programs
 from .emit import emit_header, emit_translation_unit
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -14,14 +14,17 @@ CSRC = os.path.join(_PKG, "csrc")
 GEN_DIR = os.path.join(CSRC, "build", "dsl")
 SRC_PATH = os.path.join(GEN_DIR, "tyr_dsl_kernels.hip")
 LIB_PATH = os.path.join(_PKG, "lib", "libtyr_dsl.so")
+# the statement-coverage programs of op_programs.py, used by the tests only
+OPS_SRC_PATH = os.path.join(GEN_DIR, "tyr_dsl_ops.hip")
+OPS_LIB_PATH = os.path.join(_PKG, "lib", "libtyr_dsl_ops.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
             "-packed-fp32-ops"]
 
 
-def emit_sources(path: str = SRC_PATH) -> str:
+def emit_sources(path: str = SRC_PATH, programs=kernels.ALL) -> str:
     os.makedirs(os.path.dirname(path), exist_ok=True)
-    src = emit_translation_unit([f() for f in kernels.ALL])
+    src = emit_translation_unit([f() for f in programs])
     with open(path, "w") as f:
         f.write(src)
     return path
@@ -34,8 +37,7 @@ def header_text() -> str:
     return emit_header([f() for f in kernels.ALL], kernels.CITES)
 
 
-def build(lib_path: str = LIB_PATH) -> str:
-    src = emit_sources()
+def _compile(src: str, lib_path: str) -> str:
     os.makedirs(os.path.dirname(lib_path), exist_ok=True)
     cmd = [HIPCC] + HIPFLAGS + ["-I", CSRC, "-shared", src, "-o", lib_path]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -44,8 +46,17 @@ def build(lib_path: str = LIB_PATH) -> str:
     return lib_path
 
 
+def build(lib_path: str = LIB_PATH) -> str:
+    return _compile(emit_sources(), lib_path)
+
+
+def build_op_programs(lib_path: str = OPS_LIB_PATH) -> str:
+    return _compile(emit_sources(OPS_SRC_PATH, op_programs.ALL), lib_path)
+
+
 if __name__ == "__main__":
     with open(HEADER_PATH, "w") as f:
         f.write(header_text())
     print(HEADER_PATH)
     print(build())
+    print(build_op_programs())

@@ -87,6 +87,11 @@ class SoftmaxState:  # Macros.lean:86-99
     scale: RV
 
 
+def _vid(x) -> VarId:
+    """VarId of a typed handle (KVal, KIdx, ...) or the VarId itself."""
+    return x if isinstance(x, VarId) else x.id
+
+
 class KernelBuilder:
     def __init__(self, name: str, arch: str = "GFX950"):
         self.name, self.arch = name, arch
@@ -187,6 +192,9 @@ class KernelBuilder:
 
     def getBlockIdxZ(self) -> VarId:
         v = self.freshVar(); self.emit(stmt("getBlockIdx", v, 2)); return v
+
+    def getThreadIdxX(self) -> VarId:
+        v = self.freshVar(); self.emit(stmt("getThreadIdx", v, 0)); return v
 
     def constIntVal(self, value: int) -> VarId:
         v = self.freshVar(); self.emit(stmt("constInt", v, int(value))); return v
@@ -366,6 +374,80 @@ class KernelBuilder:
         finally:
             body = self._stack.pop()
             self.emit(stmt("forLoop", v, lo, hi, body))
+
+    # ---- Loop.lean:68, 142-145: `for i in kvrange lo n do body` with a runtime bound
+    @contextlib.contextmanager
+    def kvrange(self, lo: int, hi):
+        v = self.freshVar()
+        self._stack.append([])
+        try:
+            yield KIdx(v)
+        finally:
+            body = self._stack.pop()
+            self.emit(stmt("forLoopVal", v, lo, _vid(hi), body))
+
+    # ---- IR.lean:179 ifStmt.  `with k.ifThen(c): ...` then optionally `with k.orElse(): ...` right after it
+    @contextlib.contextmanager
+    def ifThen(self, cond):
+        self._stack.append([])
+        try:
+            yield
+        finally:
+            body = self._stack.pop()
+            self.emit(stmt("ifStmt", _vid(cond), body, []))
+
+    @contextlib.contextmanager
+    def orElse(self):
+        last = self._stack[-1][-1]
+        assert last.op == "ifStmt" and not last.elseBody, "orElse follows an ifThen block"
+        self._stack.append([])
+        try:
+            yield
+        finally:
+            body = self._stack.pop()
+            self._stack[-1][-1] = stmt("ifStmt", last.cond, list(last.thenBody), body)
+
+    # ---- Ops.lean:132-227 runtime scalars
+    def constFloatVal(self, value: float, name: str = "const_f") -> KVal:
+        v = self.freshVar(); self.emit(stmt("constFloat", v, float(value))); return KVal(v, "Float32", name)
+
+    def loadFloat32Scalar(self, src: GPtr, offset, name: str = "load_f32") -> KVal:
+        v = self.freshVar(); self.emit(stmt("loadScalarGlobal", v, src.id, _vid(offset))); return KVal(v, "Float32", name)
+
+    def storeFloat32Scalar(self, dst: GPtr, offset, src):
+        self.emit(stmt("storeScalarGlobal", dst.id, _vid(src), _vid(offset)))
+
+    def scalarUnary(self, op: str, src, name: str = "scalar_unary") -> KVal:
+        v = self.freshVar(); self.emit(stmt("scalarUnary", op, v, _vid(src))); return KVal(v, "Float32", name)
+
+    def scalarCompare(self, op: str, a, b, name: str = "scalar_cmp") -> KVal:
+        v = self.freshVar(); self.emit(stmt("scalarCompare", op, v, _vid(a), _vid(b))); return KVal(v, "Bool", name)
+
+    def scalarBinary(self, op: str, a, b, name: str = "scalar_binary") -> KVal:
+        v = self.freshVar(); self.emit(stmt("scalarBinary", op, v, _vid(a), _vid(b)))
+        return KVal(v, getattr(a, "scalarTy", "UInt32"), name)
+
+    def scalarSelect(self, cond, ifTrue, ifFalse, name: str = "scalar_select") -> KVal:
+        v = self.freshVar(); self.emit(stmt("scalarSelect", v, _vid(cond), _vid(ifTrue), _vid(ifFalse)))
+        return KVal(v, getattr(ifTrue, "scalarTy", "UInt32"), name)
+
+    def iotaVec(self, dst: RV, start: float = 0.0, step: float = 1.0):
+        self.emit(stmt("vecIota", dst.id, float(start), float(step)))
+
+    def fillVecScalar(self, dst: RV, scalar):
+        self.emit(stmt("vecFillScalar", dst.id, _vid(scalar)))
+
+    # ---- Ops.lean:912-938 dimensions of a global layout
+    def layoutDim(self, src: GPtr, axis: str, name: str = "layout_dim") -> KVal:
+        v = self.freshVar(); self.emit(stmt("layoutDim", v, src.id, axis)); return KVal(v, "UInt32", name)
+
+    def layoutBatch(self, src): return self.layoutDim(src, "Batch", "batch")
+    def layoutDepth(self, src): return self.layoutDim(src, "Depth", "depth")
+    def layoutRows(self, src): return self.layoutDim(src, "Rows", "rows")
+    def layoutCols(self, src): return self.layoutDim(src, "Cols", "cols")
+
+    def upperRightFill(self, dst, src, row: int, col: int, fillVal: Optional[float] = None):
+        self.emit(stmt("mask", ("UpperRightFill", int(row), int(col)), dst.id, src.id, fillVal))
 
     # ---- Macros.lean:101-163 online softmax
     def allocSoftmaxState(self, dtype, rows) -> SoftmaxState:

@@ -42,8 +42,7 @@ NVIDIA_ONLY = {"declSemaphore", "loadAsync", "storeAsync", "storeAdd", "storeAdd
                "tmaExpect", "tmaLoad", "tmaStore", "loadGlobalAsync", "storeGlobalAsync", "storeGlobalAdd",
                "storeVecGlobalAdd", "storeVecGlobalAddCoord", "multimemLoadReduce", "multimemStore", "multimemRed",
                "tcgen05Mma", "cpAsyncLoad", "tmaLoadAsync", "arrive", "arriveAndWait", "namedBarrierSync",
-               "namedBarrierArrive", "warpGroupIdx", "electOneSync", "semaphore", "ifWarpGroup", "cumsum", "cumprod",
-               "vecIota", "vecFillScalar"}
+               "namedBarrierArrive", "warpGroupIdx", "electOneSync", "semaphore", "ifWarpGroup", "cumsum", "cumprod"}
 
 
 def _cpp_type(dtype: str) -> str:
@@ -206,6 +205,9 @@ class _Emitter:
             return f"{ind}wave::convert({I(s.dst)}, {I(s.src)});\n"
         if op == "mask":
             tag = s.args[0]
+            if tag[0] == "UpperRightFill":
+                fill = _flt(0.0 if s.fillVal is None else s.fillVal)
+                return f"{ind}wave::mask_upper_right({I(s.dst)}, {I(s.src)}, {fill}, {tag[1]}, {tag[2]});\n"
             if tag[0] not in MASK:
                 raise UnsupportedStatement(f"mask {tag[0]} has no gfx950 lowering yet")
             fill = _flt(0.0 if s.fillVal is None else s.fillVal)
@@ -256,6 +258,10 @@ class _Emitter:
             return f"{ind}const auto {I(s.dst)} = {e};\n"
         if op == "scalarSelect":
             return f"{ind}const auto {I(s.dst)} = {I(s.cond)} ? {I(s.ifTrue)} : {I(s.ifFalse)};\n"
+        if op == "vecIota":
+            return f"{ind}wave::iota({I(s.dst)}, {_flt(s.start)}, {_flt(s.step)});\n"
+        if op == "vecFillScalar":
+            return f"{ind}wave::fill({I(s.dst)}, (float){I(s.scalar)});\n"
         if op == "raw":
             return f"{ind}{s.code}\n"
         raise UnsupportedStatement(op)

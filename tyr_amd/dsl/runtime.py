@@ -7,31 +7,35 @@ from __future__ import annotations
 import ctypes
 import os
 
-from .build import LIB_PATH
+from .build import LIB_PATH, OPS_LIB_PATH
 from .ir import Kernel
 
-_lib = None
+_libs = {}
 _CT = {"UInt8": ctypes.c_uint8, "UInt16": ctypes.c_uint16, "UInt32": ctypes.c_uint32, "UInt64": ctypes.c_uint64,
        "USize": ctypes.c_size_t, "Float": ctypes.c_double, "Float32": ctypes.c_float, "Bool": ctypes.c_uint8}
 _TORCH_DTYPE = {"Float32": "float32", "BFloat16": "bfloat16", "Float16": "float16"}
 
 
-def load() -> ctypes.CDLL:
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m tyr_amd.dsl.build`. "
+def load(path: str = LIB_PATH) -> ctypes.CDLL:
+    if path not in _libs:
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python -m tyr_amd.dsl.build`. "
                                "Emitted kernels have no CPU fallback.")
-        _lib = ctypes.CDLL(LIB_PATH)
-    return _lib
+        _libs[path] = ctypes.CDLL(path)
+    return _libs[path]
 
 
-def launch(kernel: Kernel, args, grid=(1, 1, 1), block=(128, 1, 1), shared_mem: int = 0, stream=None) -> None:
+def load_op_programs() -> ctypes.CDLL:
+    return load(OPS_LIB_PATH)
+
+
+def launch(kernel: Kernel, args, grid=(1, 1, 1), block=(128, 1, 1), shared_mem: int = 0, stream=None,
+           library: ctypes.CDLL = None) -> None:
     """args: one entry per kernel parameter, in order -- a CUDA tensor for a pointer, a number for a scalar."""
     import torch
     if len(args) != len(kernel.params):
         raise TypeError(f"{kernel.name} takes {len(kernel.params)} arguments, got {len(args)}")
-    fn = getattr(load(), f"tyr_launch_{kernel.name}")
+    fn = getattr(library if library is not None else load(), f"tyr_launch_{kernel.name}")
     cargs, ctypes_sig, keep = [], [], []
     for p, a in zip(kernel.params, args):
         if p.isPointer:
