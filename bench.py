@@ -316,10 +316,11 @@ def wl_layernorm(torch, tyr, steps, warmup, cpu):
     res = _hbm_result("layernorm GB/s", "fused residual + LayerNorm, bf16, 65536 rows of 1024",
                       "layernorm_residual_kernel<2>", nbytes, ms, wall, "f32 arithmetic on bf16 data")
     if cpu:
-        xc, rc = (t[:4096].cpu() for t in xs[0])
-        dt, reps = _cpu_time(lambda: lt.layer_norm_residual(xc, rc, w.cpu(), b.cpu(), 1e-5))
-        res["cpu_baseline"] = {"value": nbytes / 16 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"LibTorch CPU add + layer_norm on 4096 of 65536 rows, {reps} reps, {dt * 1e3:.0f} ms each"}
+        xc, rc = (t.cpu() for t in xs[0])            # all rows: a slice that fits the host caches would flatter the CPU
+        wc, bc = w.cpu(), b.cpu()
+        dt, reps = _cpu_time(lambda: lt.layer_norm_residual(xc, rc, wc, bc, 1e-5))
+        res["cpu_baseline"] = {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"LibTorch CPU add + layer_norm on all 65536 rows, {reps} reps, {dt * 1e3:.1f} ms each"}
     return res
 
 
