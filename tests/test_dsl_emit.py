@@ -195,3 +195,29 @@ def test_statement_coverage_programs_lower_and_are_built():
     L = runtime.load_op_programs()
     for f in op_programs.ALL:
         assert hasattr(L, f"tyr_launch_{f().name}")
+
+
+def test_write_after_read_hazards_on_shared_tiles_get_barriers():
+    # LayerNorm reuses one LDS tile for x, residual and the output without barriers between a read
+    # and the next overwrite (the reference launches it with one warp for that reason); the emitter
+    # closes exactly those gaps, also across the loop back-edge, and adds nothing where the program
+    # already synchronises
+    src = dsl.emit_kernel(kernels.tkFusedLayerNormResidual1024())
+    assert src.count("// inserted:") == 5
+    loop = src[src.index("Pass 1"):src.index("Pass 2")]
+    first = loop[loop.index("{"):]
+    assert first.lstrip("{\n ").startswith("wave::sync();  // inserted")      # back-edge: tile read at the end of the previous pass
+    assert dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse()).count("// inserted:") == 0
+    assert dsl.emit_kernel(kernels.tkFusedLayerNormResidual1024(), hazard_barriers=False).count("// inserted:") == 0
+    # a conditional cannot hold a barrier: it goes in front of the conditional
+    k = dsl.KernelBuilder("cond")
+    g = k.gptr("Float32", "g")
+    c = k.blockCoord2D()
+    t = k.allocRT("Float32", 64, 64)
+    s_ = k.allocST("Float32", 64, 64)
+    k.loadGlobal(s_, g, c)
+    k.load(t, s_)
+    with k.ifThen(k.scalarCompare("Eq", c.r, c.c)):
+        k.store(s_, t)
+    text = dsl.emit_kernel(k.build())
+    assert text.index("// inserted:") < text.index("if (")

@@ -48,8 +48,9 @@ def test_rotaryFwd(rt):
     assert float((out.cpu() - torch.from_numpy(want)).abs().max()) <= 1e-6
 
 
+@pytest.mark.parametrize("block", [32, 128])     # the runner's single warp, and four waves sharing the LDS tile
 @pytest.mark.parametrize("rows", [64, 192])
-def test_tkFusedLayerNormResidual1024(rt, rows):
+def test_tkFusedLayerNormResidual1024(rt, rows, block):
     kernels, runtime = rt
     g = torch.Generator().manual_seed(rows)
     x = torch.rand(1, rows, 1024, generator=g).bfloat16()
@@ -60,7 +61,7 @@ def test_tkFusedLayerNormResidual1024(rt, rows):
                                                      bits(w), bits(b), 1e-5)
     out, out_resid = torch.zeros_like(x).cuda(), torch.zeros_like(x).cuda()
     runtime.launch(kernels.tkFusedLayerNormResidual1024(), [x.cuda(), res.cuda(), w.cuda(), b.cuda(), out, out_resid],
-                   grid=(1, rows // 64, 1), block=(32, 1, 1))            # the runner's single-warp launch
+                   grid=(1, rows // 64, 1), block=(block, 1, 1))
     torch.cuda.synchronize()
     got_out, got_resid = out.cpu().float().reshape(rows, 1024), out_resid.cpu().float().reshape(rows, 1024)
     assert torch.allclose(got_resid, from_bits(want_resid).float(), rtol=1e-5, atol=1e-5)
@@ -109,3 +110,44 @@ def test_launcher_rejects_bad_arguments(rt):
         runtime.launch(kernels.copy64x64(), [x, torch.zeros(1, 1, 1, 64, 64).cuda()])
     with pytest.raises(RuntimeError, match="invalid launch arguments"):
         runtime.launch(kernels.copy64x64(), [x, x.clone()], block=(1024, 1, 1))
+
+
+def test_mha_h100_forward_prep_and_backward_programs(rt):
+    """The sequence of Examples/GPU/RunMhaH100.lean:103-147 on q, k, v, dO [1,1,128,64]: both forward
+    programs agree on L = -8 LSE, the prep program gives d = rowsum(dO * O), the backward program gives
+    dQ and per-(kv tile, q tile) partials of dK and dV that are summed over q tiles on the host; all
+    against the float64 checker at the runner's allclose(3e-2, 3e-2)."""
+    kernels, runtime = rt
+    q, k, v, dO = lt.make_inputs(21, (1, 1, 128, 64), (1, 1, 128, 64), (1, 1, 128, 64), (1, 1, 128, 64))
+    geo = dict(grid=(1, 2, 1), block=(128, 1, 1))
+    qc, kc, vc, dOc = (t.cuda() for t in (q, k, v, dO))
+
+    out_lse, lse = torch.zeros_like(qc), torch.zeros(2, 64).cuda()
+    runtime.launch(kernels.tkFlashAttnFwd2BlockLse(), [qc, kc, vc, out_lse, lse, 128, 64], **geo)
+    out_plain = torch.zeros_like(qc)
+    runtime.launch(kernels.tkFlashAttnFwd2Block(), [qc, kc, vc, out_plain, 128, 64], **geo)
+    out, l_out = torch.zeros_like(qc), torch.zeros(2, 64).cuda()
+    runtime.launch(kernels.tkMhaH100Fwd2Block(), [qc, kc, vc, out, l_out, 128, 64], **geo)
+    d_vec = torch.zeros(2, 64).cuda()
+    runtime.launch(kernels.tkMhaH100BwdPrep2Block(), [dOc, out, d_vec, 128, 64], **geo)
+    dQ = torch.zeros(1, 1, 128, 64).cuda()
+    dK_part, dV_part = torch.zeros(1, 1, 128, 128).cuda(), torch.zeros(1, 1, 128, 128).cuda()
+    runtime.launch(kernels.tkMhaH100Bwd2BlockPartials(), [qc, kc, vc, dOc, l_out, d_vec, dQ, dK_part, dV_part, 128, 64],
+                   **geo)
+    torch.cuda.synchronize()
+    dK = dK_part.reshape(1, 1, 2, 64, 2, 64).sum(4).reshape(1, 1, 128, 64).cpu()
+    dV = dV_part.reshape(1, 1, 2, 64, 2, 64).sum(4).reshape(1, 1, 128, 64).cpu()
+
+    want_o, want_lse = oracle.attn_fwd_f64(bits(q), bits(k), bits(v), False, 0.125)
+    want_dq, want_dk, want_dv = oracle.attn_bwd_f64(bits(q), bits(k), bits(v), bits(dO), False, 0.125)
+    T = torch.from_numpy
+    close = lambda a, b: torch.allclose(a.cpu().float(), b.float(), rtol=3e-2, atol=3e-2)
+    assert torch.equal(out, out_lse) and torch.equal(out, out_plain)          # the three forwards share their O path
+    assert close(out, T(want_o))
+    assert close(l_out.reshape(128), -8.0 * T(want_lse).reshape(128))
+    assert torch.allclose(l_out, -8.0 * lse, rtol=0, atol=1e-5)                # the runner's cross-check of the two L paths
+    want_d = (dO.float() * out.cpu().float()).sum(-1).reshape(2, 64)
+    assert torch.allclose(d_vec.cpu(), want_d, rtol=1e-5, atol=1e-5)
+    assert close(dQ, T(want_dq)) and close(dK, T(want_dk)) and close(dV, T(want_dv))
+    for got, want in ((dQ.cpu(), T(want_dq)), (dK, T(want_dk)), (dV, T(want_dv))):
+        assert float((got.double() - want.double()).norm() / want.double().norm()) <= 1e-2

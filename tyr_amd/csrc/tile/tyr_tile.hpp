@@ -386,6 +386,14 @@ __device__ __forceinline__ void transpose(rt<T, C, R, layout::row>& dst, const r
 #pragma unroll
             for (int s = 0; s < 16; ++s) dst.data[cb][rb][s] = src.data[rb][cb][s];
 }
+// Transpose that keeps the layout kind: through an LDS tile of the source's shape.
+template <typename T, int R, int C, layout L>
+__device__ __forceinline__ void transpose(rt<T, C, R, L>& dst, const rt<T, R, C, L>& src, st<T, R, C>& scratch) {
+    store(scratch, src);
+    typedef rt<T, C, R, L> RT;
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *scratch.at(col_of<L>(cb, s), row_of<L>(rb, s));
+    wave_fence();
+}
 // Same matrix, other layout: through an LDS tile the caller provides.
 template <typename T, int R, int C, layout LD, layout LS>
 __device__ __forceinline__ void swap_layout(rt<T, R, C, LD>& dst, const rt<T, R, C, LS>& src, st<T, R, C>& scratch) {

@@ -111,9 +111,75 @@ def infer_rv_layouts(kernel: Kernel) -> Dict[VarId, str]:
     return out
 
 
+def shared_hazard_barriers(kernel: Kernel) -> set:
+    """ids of the statements that need a workgroup barrier in front of them.
+
+    Every wave of a workgroup runs the whole tile program, so the LDS tiles and vectors are shared
+    by waves that drift apart between barriers.  Overwriting one of them while another wave may still
+    be reading its previous contents is a write-after-read hazard; the reference's programs leave
+    several of those to timing (and launch a single warp where it matters,
+    Examples/GPU/RunLayerNorm.lean:66-67).  Here the emitter closes them: a barrier goes in front of
+    any statement that overwrites a shared object read since the last barrier, loop back-edges
+    included.  (Read-after-write needs nothing: all waves write identical data and a wave reads
+    after its own write.)  A conditional body cannot hold a barrier, so the barrier goes in front of
+    the conditional."""
+    shared = {s.v for s in walk(kernel.body) if s.op in ("declST", "declSV")}
+
+    def rw(s: Stmt):
+        if s.op == "load":
+            return ({s.src} & shared, set())
+        if s.op == "store":
+            return (set(), {s.dst} & shared)
+        if s.op in ("loadGlobal", "loadVecGlobal", "loadVecGlobalCoord"):
+            return (set(), {s.dst} & shared)
+        if s.op in ("storeGlobal", "storeVecGlobal", "storeVecGlobalCoord"):
+            return ({s.src} & shared, set())
+        if s.op == "swapLayout" or (s.op == "transpose"):
+            return ({("scratch", id(s))}, {("scratch", id(s))})      # the statement's own staging tile
+        return (set(), set())
+
+    def all_rw(body):
+        r, w = set(), set()
+        for s in walk(body):
+            a, b = rw(s)
+            r |= a
+            w |= b
+        return r, w
+
+    marks = set()
+
+    def run(body, pending: set, mark: bool) -> set:
+        for s in body:
+            if s.op == "sync":
+                pending = set()
+            elif s.op in ("forLoop", "forLoopVal"):
+                end = run(s.body, set(pending), False)
+                end = run(s.body, pending | end, mark)               # second pass sees the back-edge
+                pending = pending | end
+            elif s.op == "ifStmt":
+                r, w = all_rw(s.thenBody + s.elseBody)
+                if w & pending:
+                    if mark:
+                        marks.add(id(s))
+                    pending = set()
+                pending = pending | r
+            else:
+                r, w = rw(s)
+                if w & pending:
+                    if mark:
+                        marks.add(id(s))
+                    pending = set()
+                pending = pending | r
+        return pending
+
+    run(kernel.body, set(), True)
+    return marks
+
+
 class _Emitter:
-    def __init__(self, kernel: Kernel, max_waves: int = 4):
+    def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True):
         self.k = kernel
+        self.barrier_before = shared_hazard_barriers(kernel) if hazard_barriers else set()
         # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
         # full 512-register file, and covers the 128-thread blocks the reference's runners launch
         self.max_waves = max_waves
@@ -196,6 +262,10 @@ class _Emitter:
         if op == "transpose":
             if s.dst == s.src:
                 raise UnsupportedStatement("in-place transpose changes the tile's type; use a second tile")
+            t, d = self.info[s.src], self.info[s.dst]
+            if t.layout == d.layout:     # same layout kind on both sides: the data really moves, through LDS
+                return (f"{ind}{{\n{ind}  __shared__ st<{_cpp_type(t.dtype)}, {t.rows}, {t.cols}> {I(s.dst)}_tr;\n"
+                        f"{ind}  wave::transpose({I(s.dst)}, {I(s.src)}, {I(s.dst)}_tr);\n{ind}}}\n")
             return f"{ind}wave::transpose({I(s.dst)}, {I(s.src)});\n"
         if op == "swapLayout":
             t = self.info[s.src]
@@ -267,7 +337,12 @@ class _Emitter:
         raise UnsupportedStatement(op)
 
     def body(self, stmts, ind: str) -> str:
-        return "".join(self.stmt(s, ind) for s in stmts)
+        out = ""
+        for s in stmts:
+            if id(s) in self.barrier_before:
+                out += f"{ind}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
+            out += self.stmt(s, ind)
+        return out
 
     # ------------------------------------------------------------------ kernel + launchers
     def param_decls(self):
@@ -403,9 +478,9 @@ def emit_header(kernels: List[Kernel], cites: Dict[str, str]) -> str:
     return out + "#ifdef __cplusplus\n}\n#endif\n\n#endif /* TYR_DSL_KERNELS_H */\n"
 
 
-def emit_kernel(kernel: Kernel) -> str:
+def emit_kernel(kernel: Kernel, hazard_barriers: bool = True) -> str:
     """Device code of one kernel (no includes)."""
-    return _Emitter(kernel).kernel_text()
+    return _Emitter(kernel, hazard_barriers=hazard_barriers).kernel_text()
 
 
 def emit_translation_unit(kernels: List[Kernel]) -> str:

@@ -223,15 +223,16 @@ def simpleGemm(numKBlocks: int = 8) -> Kernel:
     return k.build()
 
 
-def tkFlashAttnFwd2BlockLse() -> Kernel:
-    """Tyr/GPU/Kernels/MhaH100.lean:71-128 -- attention forward of one 64-row query tile over two
-    64-row KV blocks (D = 64, scale 1/8), O in bf16 and LSE = ln(l) + m in f32."""
-    k = KernelBuilder("tkFlashAttnFwd2BlockLse")
+def _flash_attn_fwd_2block(name: str, out_kind: str) -> Kernel:
+    """The three 2-block forward programs of Tyr/GPU/Kernels/MhaH100.lean share everything but their
+    second output: none (`tkFlashAttnFwd2Block`, :14-68), LSE = ln(l) + m (`tkFlashAttnFwd2BlockLse`,
+    :71-128) or L = -8 LSE, the ThunderKittens convention for D = 64 (`tkMhaH100Fwd2Block`, :130-190)."""
+    k = KernelBuilder(name)
     q_ptr = k.gptr("BFloat16", "q_ptr")
     k_ptr = k.gptr("BFloat16", "k_ptr")
     v_ptr = k.gptr("BFloat16", "v_ptr")
     o_ptr = k.gptr("BFloat16", "o_ptr")
-    lse_ptr = k.gptr("Float32", "lse_ptr")
+    vec_ptr = k.gptr("Float32", "lse_ptr" if out_kind == "lse" else "l_ptr") if out_kind != "none" else None
     k.kval("UInt64", "_seq_len")
     k.kval("UInt64", "_head_dim")
     tileSize = 64
@@ -251,7 +252,7 @@ def tkFlashAttnFwd2BlockLse() -> Kernel:
     kShared = k.allocST("BFloat16", tileSize, tileSize)
     vShared = k.allocST("BFloat16", tileSize, tileSize, "Col")
     oShared = k.allocST("BFloat16", tileSize, tileSize)
-    lseShared = k.allocSV("Float32", tileSize)
+    vecShared = k.allocSV("Float32", tileSize) if out_kind != "none" else None
 
     k.loadGlobal(qShared, q_ptr, coord)
     k.sync()
@@ -275,15 +276,183 @@ def tkFlashAttnFwd2BlockLse() -> Kernel:
         k.sync()
 
     k.finalizeSoftmax(o, softmaxState)
-    lse = k.computeLSE(softmaxState)
+    if out_kind != "none":
+        lse = k.computeLSE(softmaxState)
+        if out_kind == "l":
+            k.scalarMulVec(lse, lse, -8.0)
 
     oBf16 = k.allocRT("BFloat16", tileSize, tileSize)
     k.convert(oBf16, o)
     k.store(oShared, oBf16)
     k.storeGlobal(o_ptr, oShared, coord)
 
-    k.storeVec(lseShared, lse)
-    k.storeVecGlobalRow(lse_ptr, lseShared, coord)
+    if out_kind != "none":
+        k.storeVec(vecShared, lse)
+        k.storeVecGlobalRow(vec_ptr, vecShared, coord)
+    return k.build()
+
+
+def tkFlashAttnFwd2Block() -> Kernel:
+    return _flash_attn_fwd_2block("tkFlashAttnFwd2Block", "none")
+
+
+def tkFlashAttnFwd2BlockLse() -> Kernel:
+    return _flash_attn_fwd_2block("tkFlashAttnFwd2BlockLse", "lse")
+
+
+def tkMhaH100Fwd2Block() -> Kernel:
+    return _flash_attn_fwd_2block("tkMhaH100Fwd2Block", "l")
+
+
+def tkMhaH100BwdPrep2Block() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:192-227 -- d[row] = sum_j dO[row, j] * O[row, j]."""
+    k = KernelBuilder("tkMhaH100BwdPrep2Block")
+    dO_ptr = k.gptr("BFloat16", "dO_ptr")
+    o_ptr = k.gptr("BFloat16", "o_ptr")
+    d_ptr = k.gptr("Float32", "d_ptr")
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    tileSize = 64
+    coord = k.blockCoord2D()
+
+    dO = k.allocRT("BFloat16", tileSize, tileSize)
+    o = k.allocRT("BFloat16", tileSize, tileSize)
+    dOf = k.allocRT("Float32", tileSize, tileSize)
+    of = k.allocRT("Float32", tileSize, tileSize)
+    prod = k.allocRT("Float32", tileSize, tileSize)
+    dVec = k.allocRV("Float32", tileSize)
+
+    dOShared = k.allocST("BFloat16", tileSize, tileSize)
+    oShared = k.allocST("BFloat16", tileSize, tileSize)
+    dShared = k.allocSV("Float32", tileSize)
+
+    k.loadGlobal(dOShared, dO_ptr, coord)
+    k.loadGlobal(oShared, o_ptr, coord)
+    k.sync()
+    k.load(dO, dOShared)
+    k.load(o, oShared)
+
+    k.convert(dOf, dO)
+    k.convert(of, o)
+    k.mul(prod, dOf, of)
+    k.rowSum(dVec, prod)
+
+    k.storeVec(dShared, dVec)
+    k.storeVecGlobalRow(d_ptr, dShared, coord)
+    return k.build()
+
+
+def tkMhaH100Bwd2BlockPartials() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:229-344 -- backward of one 64-row query tile over two KV blocks
+    (non-causal): dQ final, dK / dV as one 64x64 partial per (kv tile, q tile) that the caller sums
+    over q tiles (Examples/GPU/RunMhaH100.lean:131-138).  Scores are kept in K x Q orientation."""
+    k = KernelBuilder("tkMhaH100Bwd2BlockPartials")
+    q_ptr = k.gptr("BFloat16", "q_ptr")
+    k_ptr = k.gptr("BFloat16", "k_ptr")
+    v_ptr = k.gptr("BFloat16", "v_ptr")
+    dO_ptr = k.gptr("BFloat16", "dO_ptr")
+    l_ptr = k.gptr("Float32", "l_ptr")
+    d_ptr = k.gptr("Float32", "d_ptr")
+    dQ_ptr = k.gptr("Float32", "dQ_ptr")
+    dK_part_ptr = k.gptr("Float32", "dK_part_ptr")
+    dV_part_ptr = k.gptr("Float32", "dV_part_ptr")
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    tileSize = 64
+    numKvBlocks = 2
+    scale = 0.125
+    invLScale = -0.125
+
+    coord = k.blockCoord2D()
+
+    q = k.allocRT("BFloat16", tileSize, tileSize)
+    dO = k.allocRT("BFloat16", tileSize, tileSize)
+    dQ = k.zeroRT("Float32", tileSize, tileSize)
+    lTk = k.allocRV("Float32", tileSize)
+    lse = k.allocRV("Float32", tileSize)
+    dVec = k.allocRV("Float32", tileSize)
+
+    rowShared = k.allocST("BFloat16", tileSize, tileSize)
+    colShared = k.allocST("BFloat16", tileSize, tileSize, "Col")
+    outShared = k.allocST("Float32", tileSize, tileSize)
+    vecShared = k.allocSV("Float32", tileSize)
+
+    k.loadGlobal(rowShared, q_ptr, coord)
+    k.sync()
+    k.load(q, rowShared)
+    k.loadGlobal(rowShared, dO_ptr, coord)
+    k.sync()
+    k.load(dO, rowShared)
+
+    k.loadVecGlobalRow(vecShared, l_ptr, coord)
+    k.sync()
+    k.loadVec(lTk, vecShared)
+    k.loadVecGlobalRow(vecShared, d_ptr, coord)
+    k.sync()
+    k.loadVec(dVec, vecShared)
+    k.scalarMulVec(lse, lTk, invLScale)
+
+    with k.krange(0, numKvBlocks) as kvIdx:
+        kk = k.allocRT("BFloat16", tileSize, tileSize)
+        v = k.allocRT("BFloat16", tileSize, tileSize, "Col")
+        sT = k.zeroRT("Float32", tileSize, tileSize)
+        pT = k.allocRT("Float32", tileSize, tileSize)
+        dPT = k.zeroRT("Float32", tileSize, tileSize)
+        dST = k.allocRT("Float32", tileSize, tileSize)
+        dKPart = k.zeroRT("Float32", tileSize, tileSize)
+        dVPart = k.zeroRT("Float32", tileSize, tileSize)
+
+        k.loadGlobal(rowShared, k_ptr, coord.withRow(kvIdx.id))
+        k.loadGlobal(colShared, v_ptr, coord.withRow(kvIdx.id))
+        k.sync()
+        k.load(kk, rowShared)
+        k.load(v, colShared)
+
+        k.mmaT(sT, kk, q, sT)
+        k.scalarMul(sT, sT, scale)
+        k.subRow(sT, sT, lse)
+        k.exp(pT, sT)
+
+        vRow = k.allocRT("BFloat16", tileSize, tileSize)
+        k.swapLayout(vRow, v)
+        k.mmaT(dPT, vRow, dO, dPT)
+        k.subRow(dPT, dPT, dVec)
+
+        k.mul(dST, pT, dPT)
+        dSTScaled = k.allocRT("Float32", tileSize, tileSize)
+        k.scalarMul(dSTScaled, dST, scale)
+
+        pTBf16 = k.allocRT("BFloat16", tileSize, tileSize)
+        k.convert(pTBf16, pT)
+        dSTBf16 = k.allocRT("BFloat16", tileSize, tileSize)
+        k.convert(dSTBf16, dSTScaled)
+
+        dOCol = k.allocRT("BFloat16", tileSize, tileSize, "Col")
+        k.swapLayout(dOCol, dO)
+        k.mma(dVPart, pTBf16, dOCol, dVPart)
+
+        qCol = k.allocRT("BFloat16", tileSize, tileSize, "Col")
+        k.swapLayout(qCol, q)
+        k.mma(dKPart, dSTBf16, qCol, dKPart)
+
+        dSRow = k.allocRT("BFloat16", tileSize, tileSize)
+        k.transpose(dSRow, dSTBf16)
+        kCol = k.allocRT("BFloat16", tileSize, tileSize, "Col")
+        k.swapLayout(kCol, kk)
+        k.mma(dQ, dSRow, kCol, dQ)
+
+        dkvCoord = coord.withRow(kvIdx.id).withCol(coord.r)
+        k.store(outShared, dKPart)
+        k.sync()
+        k.storeGlobal(dK_part_ptr, outShared, dkvCoord)
+        k.store(outShared, dVPart)
+        k.sync()
+        k.storeGlobal(dV_part_ptr, outShared, dkvCoord)
+        k.sync()
+
+    k.store(outShared, dQ)
+    k.sync()
+    k.storeGlobal(dQ_ptr, outShared, coord)
     return k.build()
 
 
@@ -293,6 +462,11 @@ CITES = {
     "rotaryFwd": "Tyr/GPU/Kernels/Rotary.lean:13-62 (runner Examples/GPU/RunRotary.lean:63)",
     "tkFusedLayerNormResidual1024": "Tyr/GPU/Kernels/FusedLayerNorm.lean:28-126 (runner Examples/GPU/RunLayerNorm.lean:67)",
     "simpleGemm": "Tyr/GPU/Kernels/Examples.lean:23-65",
+    "tkFlashAttnFwd2Block": "Tyr/GPU/Kernels/MhaH100.lean:14-68 (runner Examples/GPU/RunFlashAttn.lean:80)",
     "tkFlashAttnFwd2BlockLse": "Tyr/GPU/Kernels/MhaH100.lean:71-128 (runner Examples/GPU/RunFlashAttn.lean:81)",
+    "tkMhaH100Fwd2Block": "Tyr/GPU/Kernels/MhaH100.lean:130-190 (runner Examples/GPU/RunMhaH100.lean:112)",
+    "tkMhaH100BwdPrep2Block": "Tyr/GPU/Kernels/MhaH100.lean:192-227 (runner Examples/GPU/RunMhaH100.lean:119)",
+    "tkMhaH100Bwd2BlockPartials": "Tyr/GPU/Kernels/MhaH100.lean:229-344 (runner Examples/GPU/RunMhaH100.lean:126)",
 }
-ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, tkFlashAttnFwd2BlockLse)
+ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, tkFlashAttnFwd2Block, tkFlashAttnFwd2BlockLse,
+       tkMhaH100Fwd2Block, tkMhaH100BwdPrep2Block, tkMhaH100Bwd2BlockPartials)
