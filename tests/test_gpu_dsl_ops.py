@@ -152,3 +152,25 @@ def test_control_flow_and_scalars(rt, n):
     assert torch.allclose(out[:, :T].cpu(), acc[:, :T], rtol=1e-6, atol=1e-6)
     assert torch.allclose(out[:, T:].cpu(), 2.0 * acc[:, T:], rtol=1e-6, atol=1e-6)
     assert s.cpu().tolist() == [1.5, 3.0, -(1.5 * 3.0 + 1.0), float(max(n, 5) % 4), 1.5 if n >= 2 else 0.0, 42.0]
+
+
+@pytest.mark.parametrize("block", [32, 128])
+def test_scans_and_atomic_accumulation(rt, block):
+    P, runtime, L = rt
+    g = torch.Generator().manual_seed(8)
+    x = torch.rand(T, T, generator=g) * 0.2 + 0.9
+    out = torch.full((len(P.SCAN_BLOCKS) * T, T), 77.0).cuda()
+    acc0 = torch.rand(T, T, generator=g)
+    vacc0 = torch.rand(2 * T, generator=g)
+    acc, vacc = acc0.cuda(), vacc0.cuda()
+    runtime.launch(P.dslOpsScanAtomic(), [x.cuda(), out, acc, vacc], block=(block, 1, 1), library=L)
+    torch.cuda.synchronize()
+    xd = x.double()
+    want = {"cumsumRow": xd.cumsum(1), "cumsumCol": xd.cumsum(0), "cumprodRow": xd.cumprod(1), "cumprodCol": xd.cumprod(0)}
+    for i, name in enumerate(P.SCAN_BLOCKS):
+        got = out[i * T:(i + 1) * T].cpu().double()
+        assert torch.allclose(got, want[name], rtol=1e-5, atol=1e-5), name
+    waves = block // 32                                      # every wave of the workgroup adds
+    assert torch.allclose(acc.cpu(), acc0 + waves * x, rtol=1e-6, atol=1e-6)
+    rs = x.sum(1)
+    assert torch.allclose(vacc.cpu(), vacc0 + waves * torch.cat([rs, rs]), rtol=1e-5, atol=1e-5)

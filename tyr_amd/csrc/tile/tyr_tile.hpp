@@ -219,6 +219,31 @@ __device__ __forceinline__ void store(const gl<T>& dst, const sv<T, N>& src, coo
         if (lane() + 64 * k < N) *dst.at(at.b, at.d, at.r, at.c * N + lane() + 64 * k) = src.data[lane() + 64 * k];
 }
 
+// atomic accumulation into global memory (f32).  Every wave that executes the statement adds.
+template <int R, int C>
+__device__ __forceinline__ void store_add(const gl<float>& dst, const st<float, R, C>& src, coord at) {
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < R * C / 64; ++k) {
+        const int idx = lane() + 64 * k, r = idx / C, c = idx % C;
+        atomicAdd(dst.at(at.b, at.d, at.r + r, at.c + c), *src.at(r, c));
+    }
+}
+template <int N>
+__device__ __forceinline__ void store_add(const gl<float>& dst, const sv<float, N>& src, int idx) {
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) atomicAdd(dst.ptr + (size_t)idx * N + lane() + 64 * k, src.data[lane() + 64 * k]);
+}
+template <int N>
+__device__ __forceinline__ void store_add(const gl<float>& dst, const sv<float, N>& src, coord at) {
+    wave_fence();
+#pragma unroll
+    for (int k = 0; k < (N + 63) / 64; ++k)
+        if (lane() + 64 * k < N) atomicAdd(dst.at(at.b, at.d, at.r, at.c * N + lane() + 64 * k), src.data[lane() + 64 * k]);
+}
+
 // ---------------------------------------------------------------- LDS <-> registers
 template <typename T, int R, int C, layout L>
 __device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src) {
@@ -550,6 +575,66 @@ __device__ __forceinline__ void outer(rt<T, R, C, layout::row>& dst, const rv<TV
                                       const rv<TV, C, vlayout::ortho>& b) {
     typedef rt<T, R, C, layout::row> RT;
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(a.data[rb][0]) * to_f(b.data[cb][s]));
+}
+
+// ---------------------------------------------------------------- scans (ROW tiles)
+// row_scan: dst[i][j] = OP over j' <= j of src[i][j'].  A lane owns the 4-column groups 8q + 4g of
+// its row; group totals are exchanged with the other lane half and prefixed in column order.
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void row_scan(rt<T, R, C, layout::row>& dst, const rt<T, R, C, layout::row>& src) {
+    constexpr int NG = C / 8;                        // groups per lane per row
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) {
+        float v[NG][4], own[NG], other[NG];
+#pragma unroll
+        for (int k = 0; k < NG; ++k) {
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float e = to_f(src.data[rb][k >> 2][4 * (k & 3) + x]);
+                v[k][x] = x == 0 ? e : OP::f(v[k][x - 1], e);
+            }
+            own[k] = v[k][3];
+            other[k] = xor32(own[k]);
+        }
+        float base = 0.0f;
+        bool have = false;                           // `base` holds a value (no identity element is assumed)
+#pragma unroll
+        for (int k = 0; k < NG; ++k) {
+            const float lo = lg() == 0 ? own[k] : other[k], hi = lg() == 0 ? other[k] : own[k];
+            // prefix in front of this lane's group: everything before (k), plus the low half's group for the high half
+            float pre = base;
+            bool pre_have = have;
+            if (lg() == 1) { pre = have ? OP::f(base, lo) : lo; pre_have = true; }
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                dst.data[rb][k >> 2][4 * (k & 3) + x] = from_f<T>(pre_have ? OP::f(pre, v[k][x]) : v[k][x]);
+            base = have ? OP::f(OP::f(base, lo), hi) : OP::f(lo, hi);
+            have = true;
+        }
+    }
+}
+// col_scan: dst[i][j] = OP over i' <= i of src[i'][j]: a scan over the 32 lanes of a half, carried
+// from one row block to the next.
+template <typename OP, typename T, int R, int C>
+__device__ __forceinline__ void col_scan(rt<T, R, C, layout::row>& dst, const rt<T, R, C, layout::row>& src) {
+#pragma unroll
+    for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            float carry = 0.0f;
+#pragma unroll
+            for (int rb = 0; rb < R / 32; ++rb) {
+                float x = to_f(src.data[rb][cb][s]);
+#pragma unroll
+                for (int d = 1; d < 32; d <<= 1) {
+                    const float up = __shfl_up(x, d, 32);
+                    if (lr() >= d) x = OP::f(up, x);
+                }
+                if (rb > 0) x = OP::f(carry, x);
+                dst.data[rb][cb][s] = from_f<T>(x);
+                carry = __shfl(x, 31, 32);           // the block's last row, within this lane half
+            }
+        }
 }
 
 __device__ __forceinline__ void sync() { __syncthreads(); }

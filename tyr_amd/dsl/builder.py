@@ -235,6 +235,24 @@ class KernelBuilder:
     def storeVecGlobal(self, dst: GPtr, src: SV, coord: RTileCoord):
         self.emit(stmt("storeVecGlobalCoord", dst.id, src.id, coord.b, coord.d, coord.r, coord.c))
 
+    def storeGlobalAdd(self, dst: GPtr, src: ST, coord: RTileCoord):
+        self.emit(stmt("storeGlobalAdd", dst.id, src.id, coord.b, coord.d, coord.r, coord.c))
+
+    def storeVecGlobalAddRow(self, dst: GPtr, src: SV, coord: RTileCoord):
+        self.emit(stmt("storeVecGlobalAdd", dst.id, src.id, coord.r))
+
+    def storeVecGlobalAddCol(self, dst: GPtr, src: SV, coord: RTileCoord):
+        self.emit(stmt("storeVecGlobalAdd", dst.id, src.id, coord.c))
+
+    def storeVecGlobalAdd(self, dst: GPtr, src: SV, coord: RTileCoord):
+        self.emit(stmt("storeVecGlobalAddCoord", dst.id, src.id, coord.b, coord.d, coord.r, coord.c))
+
+    # ---- Ops.lean:684-700, 819-835 scans
+    def cumsumRow(self, dst: RT, src: RT): self.emit(stmt("cumsum", "Row", dst.id, src.id))
+    def cumsumCol(self, dst: RT, src: RT): self.emit(stmt("cumsum", "Col", dst.id, src.id))
+    def cumprodRow(self, dst: RT, src: RT): self.emit(stmt("cumprod", "Row", dst.id, src.id))
+    def cumprodCol(self, dst: RT, src: RT): self.emit(stmt("cumprod", "Col", dst.id, src.id))
+
     # ---- Ops.lean: products
     def mma(self, dst: RT, a: RT, b: RT, c: RT):
         self.emit(stmt("mma", "AB", dst.id, a.id, b.id, c.id))

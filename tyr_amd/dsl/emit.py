@@ -39,10 +39,10 @@ MASK = {"MakeCausal": "keep_causal", "MakeCausalT": "keep_causal_t", "Tril": "ke
         "LowerFill": "keep_lower_fill"}
 NO_OPS = {"mmaFence", "mmaCommitGroup", "mmaAsyncWait", "fenceViewAsyncShared", "fenceProxyAsync"}
 NVIDIA_ONLY = {"declSemaphore", "loadAsync", "storeAsync", "storeAdd", "storeAddAsync", "storeMinAsync", "prefetch",
-               "tmaExpect", "tmaLoad", "tmaStore", "loadGlobalAsync", "storeGlobalAsync", "storeGlobalAdd",
-               "storeVecGlobalAdd", "storeVecGlobalAddCoord", "multimemLoadReduce", "multimemStore", "multimemRed",
+               "tmaExpect", "tmaLoad", "tmaStore", "loadGlobalAsync", "storeGlobalAsync",
+               "multimemLoadReduce", "multimemStore", "multimemRed",
                "tcgen05Mma", "cpAsyncLoad", "tmaLoadAsync", "arrive", "arriveAndWait", "namedBarrierSync",
-               "namedBarrierArrive", "warpGroupIdx", "electOneSync", "semaphore", "ifWarpGroup", "cumsum", "cumprod"}
+               "namedBarrierArrive", "warpGroupIdx", "electOneSync", "semaphore", "ifWarpGroup"}
 
 
 def _cpp_type(dtype: str) -> str:
@@ -132,7 +132,8 @@ def shared_hazard_barriers(kernel: Kernel) -> set:
             return (set(), {s.dst} & shared)
         if s.op in ("loadGlobal", "loadVecGlobal", "loadVecGlobalCoord"):
             return (set(), {s.dst} & shared)
-        if s.op in ("storeGlobal", "storeVecGlobal", "storeVecGlobalCoord"):
+        if s.op in ("storeGlobal", "storeVecGlobal", "storeVecGlobalCoord", "storeGlobalAdd", "storeVecGlobalAdd",
+                    "storeVecGlobalAddCoord"):
             return ({s.src} & shared, set())
         if s.op == "swapLayout" or (s.op == "transpose"):
             return ({("scratch", id(s))}, {("scratch", id(s))})      # the statement's own staging tile
@@ -226,6 +227,20 @@ class _Emitter:
         if op in ("loadVecGlobalCoord", "storeVecGlobalCoord"):
             at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)}, (int){I(s.coordC)}}}"
             return f"{ind}wave::{'load' if op == 'loadVecGlobalCoord' else 'store'}({I(s.dst)}, {I(s.src)}, {at});\n"
+        if op == "storeGlobalAdd":
+            tile = self.info[s.src]
+            at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)} * {tile.rows}, (int){I(s.coordC)} * {tile.cols}}}"
+            return f"{ind}wave::store_add({I(s.dst)}, {I(s.src)}, {at});\n"
+        if op == "storeVecGlobalAdd":
+            return f"{ind}wave::store_add({I(s.dst)}, {I(s.src)}, (int){I(s.offset)});\n"
+        if op == "storeVecGlobalAddCoord":
+            at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)}, (int){I(s.coordC)}}}"
+            return f"{ind}wave::store_add({I(s.dst)}, {I(s.src)}, {at});\n"
+        if op in ("cumsum", "cumprod"):
+            if s.axis == "Full":
+                raise UnsupportedStatement("full scans have no gfx950 lowering")
+            f = "op_add" if op == "cumsum" else "op_mul"
+            return f"{ind}wave::{s.axis.lower()}_scan<{f}>({I(s.dst)}, {I(s.src)});\n"
         if op == "loadScalarGlobal":
             return f"{ind}const auto {I(s.dst)} = {I(s.src)}.ptr[{I(s.offset)}];\n"
         if op == "storeScalarGlobal":

@@ -281,4 +281,36 @@ def dslOpsControl() -> Kernel:
     return k.build()
 
 
-ALL = (dslOpsUnary, dslOpsBinary, dslOpsMasks, dslOpsLayout, dslOpsMma, dslOpsControl)
+SCAN_BLOCKS = ("cumsumRow", "cumsumCol", "cumprodRow", "cumprodCol")
+
+
+def dslOpsScanAtomic() -> Kernel:
+    """Scans of x (blocks of `out` in the order of SCAN_BLOCKS) and atomic accumulation: every wave of
+    the workgroup adds x to `acc` and the row sums of x to `vacc[0:64]` (row-offset form) and to
+    `vacc[64:128]` (4-D coordinate form)."""
+    k = KernelBuilder("dslOpsScanAtomic")
+    x_ptr = k.gptr("Float32", "x")
+    out = k.gptr("Float32", "out")
+    acc = k.gptr("Float32", "acc")
+    vacc = k.gptr("Float32", "vacc")
+    coord = k.blockCoord2D()
+    xs = k.allocST("Float32", T, T)
+    stage = k.allocST("Float32", T, T)
+    vs = k.allocSV("Float32", T)
+    x = k.allocRT("Float32", T, T)
+    y = k.allocRT("Float32", T, T)
+    k.loadGlobal(xs, x_ptr, coord)
+    k.load(x, xs)
+    for i, name in enumerate(SCAN_BLOCKS):
+        getattr(k, name)(y, x)
+        _emit_tile(k, out, stage, y, i)
+    k.storeGlobalAdd(acc, xs, coord)
+    v = k.allocRV("Float32", T)
+    k.rowSum(v, x)
+    k.storeVec(vs, v)
+    k.storeVecGlobalAddRow(vacc, vs, coord)
+    k.storeVecGlobalAdd(vacc, vs, coord.withCol(k.constIntVal(1)))
+    return k.build()
+
+
+ALL = (dslOpsScanAtomic, dslOpsUnary, dslOpsBinary, dslOpsMasks, dslOpsLayout, dslOpsMma, dslOpsControl)
