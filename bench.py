@@ -95,7 +95,7 @@ def wl_attn(torch, tyr, steps, warmup, cpu):
         qc, kc, vc = (t[:1, :hs].cpu() for t in (q, k, v))
         lt.sdpa_4d(qc[:, :2], kc[:, :2], vc[:, :2], True)   # warm-up
         reps, t0 = 0, time.perf_counter()
-        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 50):
+        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 400):      # about 10 s of host work
             lt.sdpa_4d(qc, kc, vc, True)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
