@@ -151,3 +151,48 @@ def test_mha_h100_forward_prep_and_backward_programs(rt):
     assert close(dQ, T(want_dq)) and close(dK, T(want_dk)) and close(dV, T(want_dv))
     for got, want in ((dQ.cpu(), T(want_dq)), (dK, T(want_dk)), (dV, T(want_dv))):
         assert float((got.double() - want.double()).norm() / want.double().norm()) <= 1e-2
+
+
+def _fp8_inputs(seed, M, N, K):
+    torch.manual_seed(seed)
+    aq, sa = lt.quantize_e4m3(torch.randn(M, K))
+    bq, sb = lt.quantize_e4m3(torch.randn(N, K))          # B is N x K (the reference's tiledAccumulator layout)
+    return aq, sa, bq, sb
+
+
+@pytest.mark.parametrize("M,N", [(64, 256), (192, 512)])
+def test_gemmFp8E4M3Fwd(rt, M, N):
+    kernels, runtime = rt
+    K = 512                                                  # 4 slices of 128
+    aq, _, bq, _ = _fp8_inputs(31, M, N, K)
+    c = torch.zeros(M, N, dtype=torch.bfloat16).cuda()
+    runtime.launch(kernels.gemmFp8E4M3Fwd(), [aq.cuda(), bq.cuda(), c, M, N, K], grid=(N // 256, M // 64, 1),
+                   block=(128, 1, 1))
+    torch.cuda.synchronize()
+    want_bits, want_f32 = oracle.gemm_fp8(aq.view(torch.uint8).numpy(), bq.view(torch.uint8).numpy(), 1.0, 1.0, trans_b=True)
+    # products of E4M3 values are exact in f32 and K = 512 terms stay far below 2^24 ulps: the f32 sums differ
+    # only by accumulation order, so nearly every bf16 output is bit-identical; the bar is the GEMM tolerance
+    got = c.cpu().float()
+    rel = float((got - torch.from_numpy(want_f32)).norm() / np.linalg.norm(want_f32))
+    assert rel <= 1e-2 and rel <= 3e-3, rel
+    want_bf, wf = from_bits(want_bits).float(), torch.from_numpy(want_f32)
+    # per element: half a bf16 ulp of rounding plus the slack of the matrix pipe's own accumulation (a 64-term dot
+    # product is aligned to its largest product before it is summed; terms reach 448^2 = 2e5)
+    assert bool(((got - wf).abs() <= wf.abs() * 2.0 ** -8 * 1.01 + 16.0).all())
+    assert float((got != want_bf).float().mean()) <= 0.05                                # bit-identical for more than 95 % of the outputs
+
+
+def test_tkH100Fp8ScaledGemmFwd(rt):
+    kernels, runtime = rt
+    M, N, K = 128, 512, 512
+    aq, _, bq, _ = _fp8_inputs(32, M, N, K)
+    g = torch.Generator().manual_seed(33)
+    sa, sb = torch.rand(M, generator=g) + 0.5, torch.rand(N, generator=g) + 0.5
+    c = torch.zeros(M, N).cuda()
+    runtime.launch(kernels.tkH100Fp8ScaledGemmFwd(), [aq.cuda(), bq.cuda(), sa.cuda(), sb.cuda(), c, M, N, K],
+                   grid=(N // 256, M // 64, 1), block=(128, 1, 1))
+    torch.cuda.synchronize()
+    _, want_f32 = oracle.gemm_fp8(aq.view(torch.uint8).numpy(), bq.view(torch.uint8).numpy(), 1.0, 1.0, trans_b=True)
+    want = torch.from_numpy(want_f32) * sa[:, None] * sb[None, :]
+    rel = float((c.cpu() - want).norm() / want.norm())
+    assert rel <= 1e-4, rel                                   # f32 accumulation order is the only difference

@@ -30,6 +30,11 @@ namespace tile {
 
 typedef __bf16 bf16;
 
+// OCP E4M3 (e4m3fn: bias 7, max 448, no infinity), one byte of storage; arithmetic happens in f32.
+struct fp8e4m3 {
+    uint8_t bits;
+};
+
 enum class layout { row, col };
 enum class vlayout { align, ortho };
 
@@ -100,6 +105,12 @@ __device__ __forceinline__ void wave_fence() {
 }
 template <typename T> __device__ __forceinline__ float to_f(T x) { return (float)x; }
 template <typename T> __device__ __forceinline__ T from_f(float x) { return (T)x; }
+template <> __device__ __forceinline__ float to_f<fp8e4m3>(fp8e4m3 x) { return __builtin_amdgcn_cvt_f32_fp8((int)x.bits, 0); }
+// round to nearest even, saturating at +-448 (the quantisation rule of the fp8 GEMM's inputs)
+template <> __device__ __forceinline__ fp8e4m3 from_f<fp8e4m3>(float x) {
+    const float c = x != x ? x : fminf(fmaxf(x, -448.0f), 448.0f);
+    return fp8e4m3{(uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(c, 0.0f, 0, false) & 0xff)};
+}
 // position of slot s of block (rb, cb) for the calling lane
 template <layout L> __device__ __forceinline__ int row_of(int rb, int s) {
     return L == layout::row ? 32 * rb + lr() : 32 * rb + 8 * (s >> 2) + 4 * lg() + (s & 3);
@@ -332,6 +343,41 @@ TYR_TILE_MMA(mma_AtB, rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA M TYR_TILE_COMMA l
 TYR_TILE_MMA(mma_AtBt, rt<bf16 TYR_TILE_COMMA K TYR_TILE_COMMA M TYR_TILE_COMMA layout::col>,
              rt<bf16 TYR_TILE_COMMA N TYR_TILE_COMMA K TYR_TILE_COMMA layout::row>, K, [kb][mb], [nb][kb])
 #undef TYR_TILE_MMA
+// E4M3 operands: A[M,K] row, B[N,K] row, on the 32x32x64 MFMA (a lane's 16 bytes of two adjacent
+// 32-column blocks are its 32 bytes of k; both operands use the same map).
+template <int M, int N, int K>
+__device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<fp8e4m3, M, K, layout::row>& a,
+                                        const rt<fp8e4m3, N, K, layout::row>& b, const rt<float, M, N, layout::row>& c) {
+    static_assert(K % 64 == 0, "E4M3 products consume k in steps of 64");
+#pragma unroll
+    for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < N / 32; ++nb) {
+            f32x16 acc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[e] = c.data[mb][nb][e];
+#pragma unroll
+            for (int kb = 0; kb < K / 32; kb += 2) {
+                i32x8 fa, fb;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int wd = 0; wd < 4; ++wd) {
+                        uint32_t ua = 0, ub = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            ua |= (uint32_t)a.data[mb][kb + h][4 * wd + e].bits << (8 * e);
+                            ub |= (uint32_t)b.data[nb][kb + h][4 * wd + e].bits << (8 * e);
+                        }
+                        fa[4 * h + wd] = (int)ua;
+                        fb[4 * h + wd] = (int)ub;
+                    }
+                acc = mfma_32x32x64_e4m3(fb, fa, acc);
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[e];
+        }
+}
 
 // ---------------------------------------------------------------- element-wise
 // Arithmetic is done in f32 whatever the storage type; results are rounded to the storage type.

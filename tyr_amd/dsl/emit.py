@@ -26,7 +26,7 @@ class LayoutConflict(ValueError):
     pass
 
 
-CPP_TYPE = {"Float32": "float", "BFloat16": "bf16"}
+CPP_TYPE = {"Float32": "float", "BFloat16": "bf16", "FP8E4M3": "fp8e4m3"}
 UNARY = {"Exp": "op_exp", "Exp2": "op_exp2", "Log": "op_log", "Log2": "op_log2", "Abs": "op_abs", "Relu": "op_relu",
          "Copy": "op_copy", "Neg": "op_neg", "Sqrt": "op_sqrt", "Rsqrt": "op_rsqrt", "Tanh": "op_tanh",
          "FastTanh": "op_tanh", "Sigmoid": "op_sigmoid", "Gelu": "op_gelu", "Silu": "op_silu", "Swish": "op_silu",

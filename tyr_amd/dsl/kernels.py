@@ -456,17 +456,99 @@ def tkMhaH100Bwd2BlockPartials() -> Kernel:
     return k.build()
 
 
+def _tiledAccumulator(k: KernelBuilder, banner, sourceNote, aPtr, bPtr, inDtype, tileM, tileK, tileN, kBlocks):
+    """Tyr/GPU/Kernels/GemmCommon.lean:22-56 -- A tile [tileM, tileK], B tile [tileN, tileK] (B is N x K),
+    f32 accumulator over kBlocks slices."""
+    k.comment(banner)
+    k.comment(sourceNote)
+    k.comment(f"Tile shape: A {tileM}x{tileK}, B {tileN}x{tileK}, C {tileM}x{tileN}")
+    coord = k.blockCoord2D()
+    a = k.allocRT(inDtype, tileM, tileK)
+    b = k.allocRT(inDtype, tileN, tileK)
+    accum = k.zeroRT("Float32", tileM, tileN)
+    aShared = k.allocST(inDtype, tileM, tileK)
+    bShared = k.allocST(inDtype, tileN, tileK)
+    with k.krange(0, kBlocks) as kBlk:
+        aCoord = coord.withCol(kBlk.id)
+        bCoord = coord.withRow(coord.c).withCol(kBlk.id)
+        k.loadGlobal(aShared, aPtr, aCoord)
+        k.loadGlobal(bShared, bPtr, bCoord)
+        k.sync()
+        k.load(a, aShared)
+        k.load(b, bShared)
+        k.mmaT(accum, a, b, accum)
+        k.sync()
+    return accum, coord
+
+
+def _h100Fp8Accumulator(k, banner, aPtr, bPtr):
+    """Tyr/GPU/Kernels/PrecisionGemm.lean:26-49 -- 64 x 256 output tile, k in 4 slices of 128."""
+    return _tiledAccumulator(k, banner, "ThunderKittens fp8_h100 tile family", aPtr, bPtr, "FP8E4M3", 64, 128, 256, 4)
+
+
+def gemmFp8E4M3Fwd() -> Kernel:
+    """Tyr/GPU/Kernels/PrecisionGemm.lean:178-189 with GemmCommon.storeConvertedTile (GemmCommon.lean:58-69):
+    E4M3 x E4M3 -> f32 -> bf16, C tile 64 x 256, K = 512."""
+    k = KernelBuilder("gemmFp8E4M3Fwd")
+    aPtr = k.gptr("FP8E4M3", "aPtr")
+    bPtr = k.gptr("FP8E4M3", "bPtr")
+    cPtr = k.gptr("BFloat16", "cPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    accum, coord = _h100Fp8Accumulator(k, "=== H100 FP8 GEMM compatibility epilogue (E4M3 -> BF16) ===", aPtr, bPtr)
+    out = k.allocRT("BFloat16", 64, 256)
+    outShared = k.allocST("BFloat16", 64, 256)
+    k.convert(out, accum)
+    k.store(outShared, out)
+    k.storeGlobal(cPtr, outShared, coord)
+    return k.build()
+
+
+def tkH100Fp8ScaledGemmFwd() -> Kernel:
+    """Tyr/GPU/Kernels/PrecisionGemm.lean:97-115 -- the same mainloop, then per-row scales of A and
+    per-column scales of B on the f32 accumulator (GemmCommon.lean:71-84, 123-133), f32 out."""
+    k = KernelBuilder("tkH100Fp8ScaledGemmFwd")
+    aPtr = k.gptr("FP8E4M3", "aPtr")
+    bPtr = k.gptr("FP8E4M3", "bPtr")
+    scaleAPtr = k.gptr("Float32", "scaleAPtr")
+    scaleBPtr = k.gptr("Float32", "scaleBPtr")
+    cPtr = k.gptr("Float32", "cPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    accum, coord = _h100Fp8Accumulator(k, "=== H100 FP8 GEMM with row/column scales ===", aPtr, bPtr)
+    scaleRowShared = k.allocSV("Float32", 64)
+    scaleColShared = k.allocSV("Float32", 256)
+    scaleRow = k.allocRV("Float32", 64)
+    scaleCol = k.allocRV("Float32", 256)
+    k.loadVecGlobalRow(scaleRowShared, scaleAPtr, coord)
+    k.loadVecGlobalCol(scaleColShared, scaleBPtr, coord)
+    k.loadVec(scaleRow, scaleRowShared)
+    k.loadVec(scaleCol, scaleColShared)
+    scaled = k.allocRT("Float32", 64, 256)
+    k.mulCol(scaled, accum, scaleRow)
+    k.mulRow(scaled, scaled, scaleCol)
+    outShared = k.allocST("Float32", 64, 256)
+    k.store(outShared, scaled)
+    k.storeGlobal(cPtr, outShared, coord)
+    return k.build()
+
+
 # kernel name -> the reference definition it restates
 CITES = {
     "copy64x64": "Tyr/GPU/Kernels/Copy.lean:16-26 (runner Examples/GPU/RunCopy.lean:28)",
     "rotaryFwd": "Tyr/GPU/Kernels/Rotary.lean:13-62 (runner Examples/GPU/RunRotary.lean:63)",
     "tkFusedLayerNormResidual1024": "Tyr/GPU/Kernels/FusedLayerNorm.lean:28-126 (runner Examples/GPU/RunLayerNorm.lean:67)",
     "simpleGemm": "Tyr/GPU/Kernels/Examples.lean:23-65",
+    "gemmFp8E4M3Fwd": "Tyr/GPU/Kernels/PrecisionGemm.lean:178-189 over GemmCommon.lean:22-69",
+    "tkH100Fp8ScaledGemmFwd": "Tyr/GPU/Kernels/PrecisionGemm.lean:97-115 over GemmCommon.lean:22-133",
     "tkFlashAttnFwd2Block": "Tyr/GPU/Kernels/MhaH100.lean:14-68 (runner Examples/GPU/RunFlashAttn.lean:80)",
     "tkFlashAttnFwd2BlockLse": "Tyr/GPU/Kernels/MhaH100.lean:71-128 (runner Examples/GPU/RunFlashAttn.lean:81)",
     "tkMhaH100Fwd2Block": "Tyr/GPU/Kernels/MhaH100.lean:130-190 (runner Examples/GPU/RunMhaH100.lean:112)",
     "tkMhaH100BwdPrep2Block": "Tyr/GPU/Kernels/MhaH100.lean:192-227 (runner Examples/GPU/RunMhaH100.lean:119)",
     "tkMhaH100Bwd2BlockPartials": "Tyr/GPU/Kernels/MhaH100.lean:229-344 (runner Examples/GPU/RunMhaH100.lean:126)",
 }
-ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, tkFlashAttnFwd2Block, tkFlashAttnFwd2BlockLse,
+ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, gemmFp8E4M3Fwd, tkH100Fp8ScaledGemmFwd,
+       tkFlashAttnFwd2Block, tkFlashAttnFwd2BlockLse,
        tkMhaH100Fwd2Block, tkMhaH100BwdPrep2Block, tkMhaH100Bwd2BlockPartials)

@@ -13,7 +13,7 @@ from .ir import Kernel
 _libs = {}
 _CT = {"UInt8": ctypes.c_uint8, "UInt16": ctypes.c_uint16, "UInt32": ctypes.c_uint32, "UInt64": ctypes.c_uint64,
        "USize": ctypes.c_size_t, "Float": ctypes.c_double, "Float32": ctypes.c_float, "Bool": ctypes.c_uint8}
-_TORCH_DTYPE = {"Float32": "float32", "BFloat16": "bfloat16", "Float16": "float16"}
+_TORCH_DTYPE = {"Float32": "float32", "BFloat16": "bfloat16", "Float16": "float16", "FP8E4M3": "float8_e4m3fn"}
 
 
 def load(path: str = LIB_PATH) -> ctypes.CDLL:
