@@ -261,6 +261,23 @@ __device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src
     typedef rt<T, R, C, L> RT;
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *src.at(row_of<L>(rb, s), col_of<L>(cb, s));
 }
+// COL tiles of 2-byte elements: a lane wants 4 consecutive rows of one column per slot group, which is
+// what the transposing LDS read delivers (16 lanes x 8 bytes along 4 rows in, 4 rows of one column out).
+template <int R, int C>
+__device__ __forceinline__ void load(rt<bf16, R, C, layout::col>& dst, const st<bf16, R, C>& src) {
+    const int i16 = lane() & 15, b16 = lane() >> 4;
+    const int srow = 4 * (b16 >> 1) + (i16 >> 2), scol = 16 * (b16 & 1) + 4 * (i16 & 3);   // this lane as a source
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bf16x4 v = ds_read_tr16(src.at(32 * rb + 8 * q + srow, 32 * cb + scol));
+#pragma unroll
+                for (int x = 0; x < 4; ++x) dst.data[rb][cb][4 * q + x] = v[x];
+            }
+}
 template <typename T, int R, int C, layout L>
 __device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, R, C, L>& src) {
     typedef rt<T, R, C, L> RT;
