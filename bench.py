@@ -53,8 +53,20 @@ def _events(torch, n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
+# The device needs some tens of milliseconds of continuous work before its clocks settle (the first
+# 50 attention launches after 10 warm-up launches run 2.5 % slower than the next 350; a 0.13 ms GEMM
+# goes from 128 to 111 us per launch over its first 15 ms).  Every workload therefore runs untimed for
+# this long before its W warm-up steps; the timed region is still exactly K steps.
+PREWARM_MS = 80.0
+
+
 def time_steps(torch, fn, steps, warmup):
-    """Runs warmup + steps launches of fn on the current stream; returns (wall ms/step, event ms/step)."""
+    """Runs the settle period, warmup + steps launches of fn on the current stream; returns (wall ms/step, event ms/step)."""
+    t_end = time.perf_counter() + PREWARM_MS * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -397,7 +409,10 @@ def main() -> int:
     ap.add_argument("--workload", default="attn_fwd_causal", choices=sorted(WORKLOADS) + sorted(CALIBRATION))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
+    ap.add_argument("--settle-ms", type=float, default=PREWARM_MS,
+                    help="untimed work before the warm-up steps of every workload, in milliseconds")
     args = ap.parse_args()
+    globals()["PREWARM_MS"] = args.settle_ms
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
         return 2
@@ -415,7 +430,8 @@ def main() -> int:
     head = {**WORKLOADS, **CALIBRATION}[args.workload](torch, tyr_amd, args.steps, args.warmup, not args.no_cpu)
     line = {
         "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms_per_step"], 5),
+        "steps": args.steps, "warmup": args.warmup, "settle_ms_before_warmup": PREWARM_MS,
+        "ms_per_step": round(head["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
         "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"), "wall_ms_per_step": round(head["wall_ms_per_step"], 5),
