@@ -144,6 +144,35 @@ __device__ __forceinline__ void load_global_to_lds_16(u32x4 rsrc, uint32_t lds_b
         : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
         : "memory");
 }
+// N consecutive kilobytes of LDS from one M0 write: the instruction's immediate offset advances the
+// LDS destination and the global source together, so request m uses immediate 1024 m and a per-lane
+// offset that has 1024 m taken off (voffset_less[m] = source offset of request m - 1024 m >= 0).
+template <int N>
+__device__ __forceinline__ void load_global_to_lds_16xN(u32x4 rsrc, uint32_t lds_base, const int (&voffset_less)[N], int soffset) {
+    static_assert(N == 2 || N == 4, "2 or 4 requests per call");
+    if constexpr (N == 4) {
+        asm volatile(
+            "s_mov_b32 m0, %0\n\t"
+            "s_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
+            "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
+            "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds"
+            :
+            : "s"(lds_base), "v"(voffset_less[0]), "v"(voffset_less[1]), "v"(voffset_less[2]), "v"(voffset_less[3]),
+              "s"(rsrc), "s"(soffset)
+            : "memory");
+    } else {
+        asm volatile(
+            "s_mov_b32 m0, %0\n\t"
+            "s_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds"
+            :
+            : "s"(lds_base), "v"(voffset_less[0]), "v"(voffset_less[1]), "s"(rsrc), "s"(soffset)
+            : "memory");
+    }
+}
 __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ds_read_b64_tr_b16: transposing LDS read.  Within each block of 16 lanes, lane 4q+p receives

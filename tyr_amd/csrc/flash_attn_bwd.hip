@@ -204,17 +204,14 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
 #pragma unroll
     for (int m = 0; m < C::PT; ++m) {
         const int row = (w * C::PT + m) * ROWS_PER_INST + lane / C::KCH;
-        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16;
+        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16 - 1024 * m;   // request m carries 1024 m as its immediate offset
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PT * 1024u);
     auto issue_kv = [&](int stage, int j0) {
         const uint32_t dst = wave_dst + (uint32_t)stage * C::TILE;
-#pragma unroll
-        for (int m = 0; m < C::PT; ++m) {
-            load_global_to_lds_16(k_rsrc, dst + m * 1024, g_voff[m], j0 * C::ROW);
-            load_global_to_lds_16(v_rsrc, dst + C::V_BASE + m * 1024, g_voff[m], j0 * C::ROW);
-        }
+        load_global_to_lds_16xN<C::PT>(k_rsrc, dst, g_voff, j0 * C::ROW);
+        load_global_to_lds_16xN<C::PT>(v_rsrc, dst + C::V_BASE, g_voff, j0 * C::ROW);
     };
 
     // row fragment (sub-tile T, k-step i): row 32T + r, chunk 2i + g
@@ -395,7 +392,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
 #pragma unroll
     for (int m = 0; m < C::PT; ++m) {
         const int row = (w * C::PT + m) * ROWS_PER_INST + lane / C::KCH;
-        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16;
+        g_voff[m] = row * C::ROW + swz<D>(row, lane % C::KCH) * 16 - 1024 * m;   // request m carries 1024 m as its immediate offset
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PT * 1024u);
@@ -411,11 +408,8 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         const bool live = jq < jq_end;
         const int soff = live ? hq * (int)head_bytes + jq * C::BQ * C::ROW : (int)(head_bytes * (uint32_t)G);
         const int ssoff = live ? (hq * npad + jq * C::BQ) * 8 : (int)(stat_bytes * (uint32_t)G);
-#pragma unroll
-        for (int m = 0; m < C::PT; ++m) {
-            load_global_to_lds_16(q_rsrc, dst + m * 1024, g_voff[m], soff);
-            load_global_to_lds_16(do_rsrc, dst + C::TILE + m * 1024, g_voff[m], soff);
-        }
+        load_global_to_lds_16xN<C::PT>(q_rsrc, dst, g_voff, soff);
+        load_global_to_lds_16xN<C::PT>(do_rsrc, dst + C::TILE, g_voff, soff);
         // every wave requests the same kilobyte of pairs (identical bytes, one instruction)
         load_global_to_lds_16(st_rsrc, lds_base + (uint32_t)stage * C::STAGE + 2 * C::TILE, lane * 16, ssoff);
     };

@@ -149,21 +149,20 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     for (int m = 0; m < C::PER_THREAD; ++m) {
         const int row = (w * C::PER_THREAD + m) * ROWS_PER_INST + lane / C::KCH;
         const int cpos = lane % C::KCH;                                 // chunk position in LDS
-        gk_voff[m] = row * C::ROW + k_swz<D>(row, cpos) * 16;          // swizzles are involutions
-        gv_voff[m] = row * C::ROW + v_swz<D>(row, cpos) * 16;
+        // (1024 m is taken off: request m carries it as its immediate offset)
+        gk_voff[m] = row * C::ROW + k_swz<D>(row, cpos) * 16 - 1024 * m;   // swizzles are involutions
+        gv_voff[m] = row * C::ROW + v_swz<D>(row, cpos) * 16 - 1024 * m;
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * C::PER_THREAD * 1024u);
 
     auto issue_k = [&](int stage, int j0) {
         const uint32_t dst = wave_dst + (uint32_t)stage * C::K_TILE;
-#pragma unroll
-        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(k_rsrc, dst + m * 1024, gk_voff[m], j0 * C::ROW);
+        load_global_to_lds_16xN<C::PER_THREAD>(k_rsrc, dst, gk_voff, j0 * C::ROW);
     };
     auto issue_v = [&](int stage, int j0) {
         const uint32_t dst = wave_dst + C::V_BASE + (uint32_t)stage * C::V_TILE;
-#pragma unroll
-        for (int m = 0; m < C::PER_THREAD; ++m) load_global_to_lds_16(v_rsrc, dst + m * 1024, gv_voff[m], j0 * C::ROW);
+        load_global_to_lds_16xN<C::PER_THREAD>(v_rsrc, dst, gv_voff, j0 * C::ROW);
     };
 
     f32x16 oacc[C::DT];

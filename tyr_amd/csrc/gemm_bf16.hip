@@ -226,33 +226,36 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K * 2, (size_t)0xffffffffu));
     const u32x4 b_rsrc = TRANS_B
         ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K * 2, (size_t)0xffffffffu))
-        : make_raw_rsrc(B + n0, (uint32_t)min(((size_t)K * N - n0) * 2, (size_t)0xffffffffu));
+        // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
+        //  off the per-lane offsets below, and those must not go negative)
+        : make_raw_rsrc(B + n0 - 1536, (uint32_t)min(((size_t)K * N - n0) * 2 + 3072, (size_t)0xffffffffu));
     int a_voff[8], b_voff[8];
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
         const int row = (w * 8 + m) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);
-        a_voff[m] = row * K * 2 + c * 16;
+        // (1024 (m % 4) is taken off: the request carries it as its immediate offset, see issue_half)
+        a_voff[m] = row * K * 2 + c * 16 - 1024 * (m & 3);
         if (TRANS_B) {
-            b_voff[m] = row * K * 2 + c * 16;
+            b_voff[m] = row * K * 2 + c * 16 - 1024 * (m & 3);
         } else {
             const int krow = (w * 8 + m) * 2 + (lane >> 5);
             const int cb = (lane & 31) ^ ((krow & 3) << 2);
-            b_voff[m] = krow * N * 2 + cb * 16;
+            b_voff[m] = krow * N * 2 + cb * 16 - 1024 * (m & 3) + 3072;
         }
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
-    // quarter q (0..3) of the requests for slice kt into stage st: 2 A + 2 B instructions
-    auto issue_quarter = [&](int st, int kt, int q) {
+    // half h (0..1) of the requests for slice kt into stage st: 4 A + 4 B instructions, each group of
+    // four behind one M0 write (the immediate offset steps the LDS destination by a kilobyte)
+    auto issue_half = [&](int st, int kt, int h) {
         const int a_soff = kt * BK * 2;
         const int b_soff = TRANS_B ? kt * BK * 2 : kt * BK * N * 2;
-        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
-#pragma unroll
-        for (int m = 2 * q; m < 2 * q + 2; ++m) {
-            load_global_to_lds_16(a_rsrc, dst + m * 1024, a_voff[m], a_soff);
-            load_global_to_lds_16(b_rsrc, dst + A_TILE + m * 1024, b_voff[m], b_soff);
-        }
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
+        const int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
+        const int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses
@@ -305,7 +308,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 
     const int KT = K / BK;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) issue_quarter(0, 0, q);
+    for (int h = 0; h < 2; ++h) issue_half(0, 0, h);
     wait_vmcnt0();
     __syncthreads();
 
@@ -321,7 +324,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         const unsigned char* St = lds + st * STAGE;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            if (s < 2) { issue_quarter(st ^ 1, kt + 1, 2 * s); issue_quarter(st ^ 1, kt + 1, 2 * s + 1); }
+            if (s < 2) issue_half(st ^ 1, kt + 1, s);
             if (s < 3) {
                 read_frags(St, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             } else {

@@ -238,19 +238,22 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K, (size_t)0xffffffffu));
     const u32x4 b_rsrc = TRANS_B
         ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K, (size_t)0xffffffffu))
-        : make_raw_rsrc(B + n0, (uint32_t)min((size_t)K * N - n0, (size_t)0xffffffffu));
+        // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
+        //  off the per-lane offsets below, and those must not go negative)
+        : make_raw_rsrc(B + n0 - 3072, (uint32_t)min((size_t)K * N - n0 + 3072, (size_t)0xffffffffu));
     int a_voff[8], b_voff[8];
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
         const int row = (w * 8 + m) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);
-        a_voff[m] = row * K + c * 16;
+        // (1024 (m % 4) is taken off: the request carries it as its immediate offset, see issue_half)
+        a_voff[m] = row * K + c * 16 - 1024 * (m & 3);
         if (TRANS_B) {
-            b_voff[m] = row * K + c * 16;
+            b_voff[m] = row * K + c * 16 - 1024 * (m & 3);
         } else {
             const int krow = (w * 8 + m) * 4 + (lane >> 4);
             const int cb = (lane & 15) ^ ((krow & 7) << 1);
-            b_voff[m] = krow * N + cb * 16;
+            b_voff[m] = krow * N + cb * 16 - 1024 * (m & 3) + 3072;
         }
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
@@ -258,12 +261,12 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     auto issue_half = [&](int st, int kt, int h) {
         const int a_soff = kt * BK;
         const int b_soff = TRANS_B ? kt * BK : kt * BK * N;
-        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
-#pragma unroll
-        for (int m = 4 * h; m < 4 * h + 4; ++m) {
-            load_global_to_lds_16(a_rsrc, dst + m * 1024, a_voff[m], a_soff);
-            load_global_to_lds_16(b_rsrc, dst + A_TILE + m * 1024, b_voff[m], b_soff);
-        }
+        // four requests behind one M0 write: the immediate offset steps the LDS destination by a kilobyte
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
+        const int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
+        const int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses.  k-step s covers bytes [64s, 64s+64) of a row; lane group g takes
