@@ -253,70 +253,70 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
         if (j < nkv_w) {
             const unsigned char* Kt = lds + (j & 1) * C::TILE;
             const unsigned char* Vt = Kt + C::V_BASE;
+            // The two 32-row sub-tiles of the tile are staggered so that the vector work of one has
+            // matrix work of the other next to it in program order: scores of T=0, then scores of T=1
+            // beside the exponentials of T=0, then the dQ products of T=0 beside the exponentials of T=1.
             f32x16 s[2], dp[2];
-#pragma unroll
-            for (int T = 0; T < 2; ++T)
+            bf16x8 dsf[4];
+            const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
+            auto scores = [&](int T) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
 #pragma unroll
-            for (int i = 0; i < C::KSTEPS; ++i) {
-#pragma unroll
-                for (int T = 0; T < 2; ++T) {
+                for (int i = 0; i < C::KSTEPS; ++i) {
                     const bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
                     s[T] = mfma_32x32x16_bf16(ka, qf[i], s[T]);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < C::KSTEPS; ++i) {
-#pragma unroll
-                for (int T = 0; T < 2; ++T) {
                     const bf16x8 va = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
                     dp[T] = mfma_32x32x16_bf16(va, dof[i], dp[T]);
                 }
-            }
-            // mask (diagonal tiles, ragged tail): register e of sub-tile T is kv row
-            // j0 + 32T + 8(e/4) + 4g + e%4
-            const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
-                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
-            if (need_mask) {
-                const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;
-                const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;
-                const int base = j0 + 4 * g;
-#pragma unroll
-                for (int T = 0; T < 2; ++T)
+            };
+            // mask (diagonal tiles, ragged tail), then dS^T = P^T o (dP^T - delta) packed into column-operand
+            // slots (group c = 2T + sh holds registers 8sh .. 8sh+7 of sub-tile T).  Register e of sub-tile T
+            // is kv row j0 + 32T + 8(e/4) + 4g + e%4.
+            auto probabilities = [&](int T) {
+                if (need_mask) {
+                    const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;
+                    const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;
+                    const int base = j0 + 4 * g;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
                         if (kv > lim || (EXT && kv < low)) s[T][e] = -INFINITY;
                     }
-            }
-            // dS^T = P^T o (dP^T - delta), packed into column-operand slots (group c = 2T + sh
-            // holds registers 8sh .. 8sh+7 of sub-tile T)
-            bf16x8 dsf[4];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int T = c >> 1, sh = c & 1;
-                u32x4 pk;
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) {
-                    const int e = 8 * sh + 2 * jj;
-                    const float p0 = fast_exp2(fmaf(s[T][e], scale_log2, -lse2));
-                    const float p1 = fast_exp2(fmaf(s[T][e + 1], scale_log2, -lse2));
-                    pk[jj] = pack_bf16(p0 * (dp[T][e] - delta), p1 * (dp[T][e + 1] - delta));
                 }
-                dsf[c] = __builtin_bit_cast(bf16x8, pk);
-            }
-            // dQ^T += K^T dS^T
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+                for (int sh = 0; sh < 2; ++sh) {
+                    u32x4 pk;
 #pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt) {
-                    const bf16x4 lo = ds_read_tr16(Kt + tr_lo[dt] + c * 16 * C::ROW);
-                    const bf16x4 hi = ds_read_tr16(Kt + tr_hi[dt] + c * 16 * C::ROW);
-                    const bf16x8 kt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const int e = 8 * sh + 2 * jj;
+                        const float p0 = fast_exp2(fmaf(s[T][e], scale_log2, -lse2));
+                        const float p1 = fast_exp2(fmaf(s[T][e + 1], scale_log2, -lse2));
+                        pk[jj] = pack_bf16(p0 * (dp[T][e] - delta), p1 * (dp[T][e + 1] - delta));
+                    }
+                    dsf[2 * T + sh] = __builtin_bit_cast(bf16x8, pk);
                 }
-            }
+            };
+            // dQ^T += K^T dS^T for the two 16-row groups of sub-tile T
+            auto accumulate = [&](int T) {
+#pragma unroll
+                for (int c = 2 * T; c < 2 * T + 2; ++c) {
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt) {
+                        const bf16x4 lo = ds_read_tr16(Kt + tr_lo[dt] + c * 16 * C::ROW);
+                        const bf16x4 hi = ds_read_tr16(Kt + tr_hi[dt] + c * 16 * C::ROW);
+                        const bf16x8 kt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
+                    }
+                }
+            };
+            scores(0);
+            scores(1);
+            probabilities(0);
+            accumulate(0);
+            probabilities(1);
+            accumulate(1);
         }
         wait_vmcnt0();
         __syncthreads();
