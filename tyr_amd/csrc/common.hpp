@@ -149,8 +149,10 @@ __device__ __forceinline__ void load_global_to_lds_16(u32x4 rsrc, uint32_t lds_b
 // offset that has 1024 m taken off (voffset_less[m] = source offset of request m - 1024 m >= 0).
 template <int N>
 __device__ __forceinline__ void load_global_to_lds_16xN(u32x4 rsrc, uint32_t lds_base, const int (&voffset_less)[N], int soffset) {
-    static_assert(N == 2 || N == 4, "2 or 4 requests per call");
-    if constexpr (N == 4) {
+    static_assert(N == 1 || N == 2 || N == 4, "1, 2 or 4 requests per call");
+    if constexpr (N == 1) {
+        load_global_to_lds_16(rsrc, lds_base, voffset_less[0], soffset);
+    } else if constexpr (N == 4) {
         asm volatile(
             "s_mov_b32 m0, %0\n\t"
             "s_nop 0\n\t"
