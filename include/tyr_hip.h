@@ -96,6 +96,17 @@ int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void
                                int causal, uint64_t window, const int32_t* kv_lens, float scale,
                                void* stream);
 
+/* The forward with an arbitrary per-sequence key mask: `lean_torch_sdpa_gqa_mask`
+ * (cc/src/tyr.cpp:4019-4095; mask [batch, seq], 1 = valid key, combined with the causal rule when
+ * is_causal) for any mask pattern, e.g. left padding.
+ *   key_mask: device uint8 [B, N]; key j of sequence b is visible iff key_mask[b*N + j] != 0.
+ * A row that sees no key gets O = 0, LSE = -inf (LibTorch returns NaN there).  Otherwise as
+ * tyr_hip_flash_attn_fwd_gqa with window = 0 and no kv_lens.
+ */
+int tyr_hip_flash_attn_fwd_mask(const void* q, const void* k, const void* v, void* o, float* lse,
+                                uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                int causal, const uint8_t* key_mask, float scale, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Flash-attention backward.
  *
@@ -165,6 +176,14 @@ int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, cons
                                uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
                                int causal, uint64_t window, const int32_t* kv_lens, float scale,
                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward of tyr_hip_flash_attn_fwd_mask (autograd of `lean_torch_sdpa_gqa_mask`,
+ * cc/src/tyr.cpp:4019-4095): hidden keys receive dk = dv = 0, rows that saw no key dq = 0. */
+int tyr_hip_flash_attn_bwd_mask(const void* q, const void* k, const void* v, const void* o,
+                                const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                                uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                int causal, const uint8_t* key_mask, float scale,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* GQA decode with a per-sequence cache length and / or a sliding window.
  *

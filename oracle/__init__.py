@@ -50,6 +50,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_attn_fwd_f64_ex.restype = None
         L.oracle_attn_bwd_f64_ex.argtypes = [vp] * 7 + [i64] * 5 + [ci, i64, vp, f64]
         L.oracle_attn_bwd_f64_ex.restype = None
+        L.oracle_attn_fwd_f64_mask.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, i64, vp, vp, f64]
+        L.oracle_attn_fwd_f64_mask.restype = None
+        L.oracle_attn_bwd_f64_mask.argtypes = [vp] * 7 + [i64] * 5 + [ci, i64, vp, vp, f64]
+        L.oracle_attn_bwd_f64_mask.restype = None
         L.oracle_attn_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f64]
         L.oracle_attn_bwd_f64.restype = None
         L.oracle_attn_fwd_tiled.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, f32, i64]
@@ -126,17 +130,20 @@ def attn_fwd_f64(q, k, v, causal: bool, scale: float):
     return o, lse
 
 
-def attn_fwd_f64_ex(q, k, v, causal: bool, scale: float, window: int = 0, kv_lens=None):
-    """Double-precision attention with grouped queries (k, v may have fewer heads), a sliding window and
-    per-sequence key lengths (int32 [B]).  -> (O f32 [B,Hq,N,D], LSE f32 [B,Hq,N])."""
+def attn_fwd_f64_ex(q, k, v, causal: bool, scale: float, window: int = 0, kv_lens=None, key_mask=None):
+    """Double-precision attention with grouped queries (k, v may have fewer heads), a sliding window,
+    per-sequence key lengths (int32 [B]) and a per-sequence key mask (uint8 / bool [B,N], nonzero = visible).
+    -> (O f32 [B,Hq,N,D], LSE f32 [B,Hq,N])."""
     q, k, v = (_chk(t, np.uint16, n) for t, n in ((q, "q"), (k, "k"), (v, "v")))
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
     o = np.empty((B, Hq, N, D), np.float32)
     lse = np.empty((B, Hq, N), np.float32)
     lens = None if kv_lens is None else _chk(np.asarray(kv_lens, dtype=np.int32), np.int32, "kv_lens")
-    lib().oracle_attn_fwd_f64_ex(_p(q), _p(k), _p(v), _p(o), _p(lse), B, Hq, Hkv, N, D, int(causal), int(window),
-                                 None if lens is None else _p(lens), float(scale))
+    km = None if key_mask is None else _chk(np.asarray(key_mask).astype(np.uint8), np.uint8, "key_mask")
+    assert km is None or km.shape == (B, N)
+    lib().oracle_attn_fwd_f64_mask(_p(q), _p(k), _p(v), _p(o), _p(lse), B, Hq, Hkv, N, D, int(causal), int(window),
+                                   None if lens is None else _p(lens), None if km is None else _p(km), float(scale))
     return o, lse
 
 
@@ -150,8 +157,8 @@ def attn_bwd_f64(q, k, v, d_o, causal: bool, scale: float):
     return dq, dk, dv
 
 
-def attn_bwd_f64_ex(q, k, v, d_o, causal: bool, scale: float, window: int = 0, kv_lens=None):
-    """Double-precision attention backward with grouped queries, window and key lengths.
+def attn_bwd_f64_ex(q, k, v, d_o, causal: bool, scale: float, window: int = 0, kv_lens=None, key_mask=None):
+    """Double-precision attention backward with grouped queries, window, key lengths and key mask.
     q, d_o uint16 [B,Hq,N,D]; k, v uint16 [B,Hkv,N,D] -> (dQ [B,Hq,N,D], dK, dV [B,Hkv,N,D]) f32."""
     q, k, v, d_o = (_chk(t, np.uint16, n) for t, n in ((q, "q"), (k, "k"), (v, "v"), (d_o, "d_o")))
     B, Hq, N, D = q.shape
@@ -159,8 +166,11 @@ def attn_bwd_f64_ex(q, k, v, d_o, causal: bool, scale: float, window: int = 0, k
     dq = np.empty((B, Hq, N, D), np.float32)
     dk, dv = np.empty((B, Hkv, N, D), np.float32), np.empty((B, Hkv, N, D), np.float32)
     lens = None if kv_lens is None else _chk(np.asarray(kv_lens, dtype=np.int32), np.int32, "kv_lens")
-    lib().oracle_attn_bwd_f64_ex(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), B, Hq, Hkv, N, D, int(causal),
-                                 int(window), None if lens is None else _p(lens), float(scale))
+    km = None if key_mask is None else _chk(np.asarray(key_mask).astype(np.uint8), np.uint8, "key_mask")
+    assert km is None or km.shape == (B, N)
+    lib().oracle_attn_bwd_f64_mask(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), B, Hq, Hkv, N, D, int(causal),
+                                   int(window), None if lens is None else _p(lens), None if km is None else _p(km),
+                                   float(scale))
     return dq, dk, dv
 
 

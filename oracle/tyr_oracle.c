@@ -25,6 +25,8 @@
  *                           dV = P^T dO, dK = scale dS^T Q, dQ = scale dS K), in
  *                           double; reference values as Examples/GPU/RunMhaH100.lean:56-64
  *                           takes them from autograd.
+ *   oracle_attn_*_f64_mask  the _ex functions with an arbitrary per-sequence key mask as well
+ *                           (cc/src/tyr.cpp:4019-4095: mask [batch, seq], 1 = valid key).
  *   oracle_attn_bwd_f64_ex  the same with grouped queries (dK / dV summed over the query
  *                           heads of a kv head: the gradient of repeat_interleave), window
  *                           and prefix key lengths.
@@ -164,9 +166,13 @@ void oracle_attn_fwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v
  * visible to query i iff j < kv_lens[b] (if given), j <= i (if causal) and i - j < window
  * (if window > 0; cc/src/tyr.cpp:3980-3996).  A row without any visible key gets O = 0,
  * LSE = -inf. */
-void oracle_attn_fwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                            float* o, float* lse, int64_t B, int64_t Hq, int64_t Hkv, int64_t N,
-                            int64_t D, int causal, int64_t window, const int32_t* kv_lens, double scale) {
+/* key_mask: uint8 [B,N], nonzero = key may be attended to (the padding mask of
+ * cc/src/tyr.cpp:4019-4095, any pattern), or NULL.  A row whose every key is hidden gives
+ * O = 0, LSE = -inf (LibTorch returns NaN there). */
+void oracle_attn_fwd_f64_mask(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                              float* o, float* lse, int64_t B, int64_t Hq, int64_t Hkv, int64_t N,
+                              int64_t D, int causal, int64_t window, const int32_t* kv_lens,
+                              const uint8_t* key_mask, double scale) {
     const int64_t G = Hq / Hkv;
     #pragma omp parallel for collapse(2) schedule(dynamic)
     for (int64_t bh = 0; bh < B * Hq; ++bh) {
@@ -190,8 +196,14 @@ void oracle_attn_fwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t
                 const uint16_t* kr = k + (kvh * N + j) * D;
                 double acc = 0.0;
                 for (int64_t d = 0; d < D; ++d) acc += (double)bf16_to_f32(qr[d]) * (double)bf16_to_f32(kr[d]);
-                s[j - jlo] = acc * scale;
+                s[j - jlo] = (key_mask && !key_mask[b * N + j]) ? -INFINITY : acc * scale;
                 if (s[j - jlo] > m) m = s[j - jlo];
+            }
+            if (m == -INFINITY) {                      /* every key in range is hidden */
+                for (int64_t d = 0; d < D; ++d) orow[d] = 0.0f;
+                if (lse) lse[bh * N + i] = -INFINITY;
+                free(s);
+                continue;
             }
             double l = 0.0;
             for (int64_t j = jlo; j < jhi; ++j) { s[j - jlo] = exp(s[j - jlo] - m); l += s[j - jlo]; }
@@ -204,6 +216,12 @@ void oracle_attn_fwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t
             free(s);
         }
     }
+}
+
+void oracle_attn_fwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                            float* o, float* lse, int64_t B, int64_t Hq, int64_t Hkv, int64_t N,
+                            int64_t D, int causal, int64_t window, const int32_t* kv_lens, double scale) {
+    oracle_attn_fwd_f64_mask(q, k, v, o, lse, B, Hq, Hkv, N, D, causal, window, kv_lens, NULL, scale);
 }
 
 /* Attention backward in double precision.  q,k,v,d_o: bf16 bit patterns [B,H,N,D];
@@ -269,10 +287,11 @@ void oracle_attn_bwd_f64(const uint16_t* q, const uint16_t* k, const uint16_t* v
  * key length (visibility rule of oracle_attn_fwd_f64_ex).  dq: f32 [B,Hq,N,D]; dk, dv: f32
  * [B,Hkv,N,D], each the sum over the Hq/Hkv query heads that read that kv head (the gradient of
  * repeat_interleave is that sum).  Rows without a visible key contribute nothing. */
-void oracle_attn_bwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                            const uint16_t* d_o, float* dq, float* dk, float* dv,
-                            int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
-                            int causal, int64_t window, const int32_t* kv_lens, double scale) {
+void oracle_attn_bwd_f64_mask(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                              const uint16_t* d_o, float* dq, float* dk, float* dv,
+                              int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                              int causal, int64_t window, const int32_t* kv_lens,
+                              const uint8_t* key_mask, double scale) {
     const int64_t G = Hq / Hkv;
     #pragma omp parallel for schedule(dynamic)
     for (int64_t bk = 0; bk < B * Hkv; ++bk) {
@@ -301,8 +320,12 @@ void oracle_attn_bwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t
                         double acc = 0.0;
                         for (int64_t d = 0; d < D; ++d)
                             acc += (double)bf16_to_f32(qh[i * D + d]) * (double)bf16_to_f32(kh[j * D + d]);
-                        p[j] = acc * scale;
+                        p[j] = (key_mask && !key_mask[b * N + j]) ? -INFINITY : acc * scale;
                         if (p[j] > m) m = p[j];
+                    }
+                    if (m == -INFINITY) {              /* every key hidden: the row contributes nothing */
+                        for (int64_t d = 0; d < D; ++d) dq[(bh * N + i) * D + d] = 0.0f;
+                        continue;
                     }
                     double l = 0.0;
                     for (int64_t j = jlo; j < jhi; ++j) { p[j] = exp(p[j] - m); l += p[j]; }
@@ -333,6 +356,13 @@ void oracle_attn_bwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t
         }
         free(dka); free(dva); free(p); free(dp); free(dqa);
     }
+}
+
+void oracle_attn_bwd_f64_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                            const uint16_t* d_o, float* dq, float* dk, float* dv,
+                            int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                            int causal, int64_t window, const int32_t* kv_lens, double scale) {
+    oracle_attn_bwd_f64_mask(q, k, v, d_o, dq, dk, dv, B, Hq, Hkv, N, D, causal, window, kv_lens, NULL, scale);
 }
 
 /* Tiled online-softmax attention in the reference kernel's order of operations:

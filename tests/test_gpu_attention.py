@@ -345,3 +345,49 @@ def test_attention_error_convention(gpu):
     with pytest.raises(TyrGpuError, match="must have dim <= 4"):
         z = torch.zeros(1, 1, 1, 16, 128, dtype=torch.bfloat16).cuda()
         gpu.flash_attn_fwd(z, z, z)
+
+
+def _scattered_key_mask(B, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    m = torch.rand(B, N, generator=g) < 0.6
+    m[0] = True                                              # one sequence without padding
+    if B > 1:
+        m[1, : N // 3] = False                               # left padding: causal rows there see no key at all
+    return m
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(3, 4, 2, 200, 128), (2, 2, 2, 129, 64), (2, 8, 1, 64, 128), (1, 1, 1, 1, 64)])
+def test_flash_attn_arbitrary_key_mask_matches_oracle(gpu, B, Hq, Hkv, N, D, causal):
+    # lean_torch_sdpa_gqa_mask (cc/src/tyr.cpp:4019-4095) with holes anywhere, left padding included
+    q, = lt.make_inputs(900 + N, (B, Hq, N, D))
+    k, v = lt.make_inputs(901 + N, (B, Hkv, N, D), (B, Hkv, N, D))
+    km = _scattered_key_mask(B, N, 902 + N)
+    sc = 1.0 / math.sqrt(D)
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc, key_mask=km.cuda())
+    want_o, want_lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, sc, key_mask=km.numpy())
+    assert max_abs(o.cpu().float(), want_o) <= 2e-2
+    dead = np.isneginf(want_lse)
+    got_lse = lse.cpu().numpy()
+    assert np.array_equal(np.isneginf(got_lse), dead)                       # rows that see no key: LSE = -inf ...
+    assert float(o.cpu().float().numpy()[dead].__abs__().max(initial=0.0)) == 0.0   # ... and O = 0
+    assert float(np.abs(got_lse[~dead] - want_lse[~dead]).max(initial=0.0)) <= 2e-2
+    # uint8 masks are the same thing, and an all-visible mask is no mask
+    o8, _ = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc, key_mask=km.to(torch.uint8).cuda())
+    assert torch.equal(o8, o)
+    o1, l1 = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc,
+                                key_mask=torch.ones(B, N, dtype=torch.bool).cuda())
+    o0, l0 = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc)
+    assert max_abs(o1.cpu().float(), o0.cpu().float()) <= 1e-2 and max_abs(l1.cpu(), l0.cpu()) <= 1e-3
+
+
+def test_flash_attn_key_mask_argument_checks(gpu):
+    q, k, v = (t.cuda() for t in lt.make_inputs(5, (1, 2, 64, 64), (1, 2, 64, 64), (1, 2, 64, 64)))
+    with pytest.raises(gpu.TyrGpuError, match="shape"):
+        gpu.flash_attn_fwd(q, k, v, key_mask=torch.ones(1, 63, dtype=torch.bool).cuda())
+    with pytest.raises(gpu.TyrGpuError, match="dtype"):
+        gpu.flash_attn_fwd(q, k, v, key_mask=torch.ones(1, 64).cuda())
+    with pytest.raises(gpu.TyrGpuError, match="CUDA"):
+        gpu.flash_attn_fwd(q, k, v, key_mask=torch.ones(1, 64, dtype=torch.bool))
+    with pytest.raises(gpu.TyrGpuError, match="combined"):
+        gpu.flash_attn_fwd(q, k, v, window=4, key_mask=torch.ones(1, 64, dtype=torch.bool).cuda())

@@ -151,3 +151,27 @@ def test_flash_attn_bwd_error_convention(gpu):
     b = torch.zeros(1, 1, 16, 96, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(gpu.TyrGpuError, match="not supported"):
         gpu.flash_attn_bwd(b, b, b, b, lse, b)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(3, 4, 2, 200, 128), (2, 2, 2, 129, 64), (2, 8, 1, 300, 128)])
+def test_flash_attn_bwd_arbitrary_key_mask(gpu, B, Hq, Hkv, N, D, causal):
+    # autograd of lean_torch_sdpa_gqa_mask (cc/src/tyr.cpp:4019-4095) with holes anywhere and left padding
+    q, g = lt.make_inputs(8300 + N, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(8301 + N, (B, Hkv, N, D), (B, Hkv, N, D))
+    gen = torch.Generator().manual_seed(8302 + N)
+    km = torch.rand(B, N, generator=gen) < 0.6
+    km[0] = True
+    km[1, : N // 3] = False
+    sc = 1 / math.sqrt(D)
+    qd, kd, vd, gd, kmd = (t.cuda() for t in (q, k, v, g, km))
+    o, lse = gpu.flash_attn_fwd(qd, kd, vd, causal=causal, scale=sc, key_mask=kmd)
+    dq, dk, dv = gpu.flash_attn_bwd(qd, kd, vd, o, lse, gd, causal=causal, scale=sc, key_mask=kmd)
+    wq, wk, wv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), causal, sc, key_mask=km.numpy())
+    check(dq, wq, "dq")
+    check(dk, wk, "dk")
+    check(dv, wv, "dv")
+    hidden = ~km.unsqueeze(1).expand(B, Hkv, N)           # hidden keys get no gradient at all
+    assert float(dk.cpu().float()[hidden].abs().max()) == 0.0 and float(dv.cpu().float()[hidden].abs().max()) == 0.0
+    if causal:                                            # left-padded rows that saw no key: dQ = 0
+        assert float(dq[1, :, : N // 3].float().abs().max()) == 0.0

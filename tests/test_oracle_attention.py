@@ -231,3 +231,51 @@ def test_f64_ex_key_lengths_match_libtorch_padding_mask(causal):
     v2[1, :, 7:] = -9.0
     o2, _ = oracle.attn_fwd_f64_ex(bits(q), bits(k2), bits(v2), causal, 0.25, kv_lens=lens)
     np.testing.assert_array_equal(o, o2)
+
+
+def _scattered_mask(B, N, seed, keep_first):
+    g = torch.Generator().manual_seed(seed)
+    m = (torch.rand(B, N, generator=g) < 0.6)
+    if keep_first:
+        m[:, 0] = True                              # causal row 0 then sees a key (LibTorch gives NaN otherwise)
+    m[0] = True                                     # one sequence without padding
+    return m
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_f64_ex_arbitrary_key_mask_matches_libtorch_padding_mask(causal):
+    # lean_torch_sdpa_gqa_mask with a mask that is not a prefix: holes anywhere in the sequence
+    B, Hq, Hkv, N, D = 3, 4, 2, 70, 16
+    q, = lt.make_inputs(41, (B, Hq, N, D))
+    k, v = lt.make_inputs(42, (B, Hkv, N, D), (B, Hkv, N, D))
+    km = _scattered_mask(B, N, 43, keep_first=True)
+    o, lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25, key_mask=km.numpy())
+    ref = lt.sdpa_gqa_mask(q.double(), k.double(), v.double(), km.long(), causal)
+    np.testing.assert_allclose(o, ref.numpy(), atol=1e-5)
+    # a hidden key's contents do not matter; an all-visible mask is no mask; a prefix mask is a key length
+    k2, v2 = k.clone(), v.clone()
+    k2[~km.unsqueeze(1).expand(B, Hkv, N)] = 7.0
+    v2[~km.unsqueeze(1).expand(B, Hkv, N)] = -7.0
+    o2, lse2 = oracle.attn_fwd_f64_ex(bits(q), bits(k2), bits(v2), causal, 0.25, key_mask=km.numpy())
+    np.testing.assert_array_equal(o, o2)
+    np.testing.assert_array_equal(lse, lse2)
+    o3, _ = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25, key_mask=np.ones((B, N), np.uint8))
+    o4, _ = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25)
+    np.testing.assert_array_equal(o3, o4)
+    lens = [70, 9, 31]
+    pm = (torch.arange(N)[None, :] < torch.tensor(lens)[:, None])
+    o5, l5 = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25, key_mask=pm.numpy())
+    o6, l6 = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, 0.25, kv_lens=lens)
+    np.testing.assert_array_equal(o5, o6)
+    np.testing.assert_array_equal(l5, l6)
+
+
+def test_f64_ex_row_with_every_key_hidden_is_zero():
+    B, H, N, D = 1, 1, 12, 16
+    q, k, v = lt.make_inputs(44, (B, H, N, D), (B, H, N, D), (B, H, N, D))
+    km = np.ones((B, N), np.uint8)
+    km[0, :3] = 0                                   # causal rows 0..2 see nothing
+    o, lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), True, 0.25, key_mask=km)
+    assert np.all(o[0, 0, :3] == 0) and np.all(np.isneginf(lse[0, 0, :3]))
+    assert np.all(np.isfinite(lse[0, 0, 3:]))
+    np.testing.assert_allclose(o[0, 0, 3], v[0, 0, 3].float().numpy(), atol=1e-6)      # row 3 sees only key 3

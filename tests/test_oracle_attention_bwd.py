@@ -144,3 +144,25 @@ def test_bwd_ex_reduces_to_plain_backward():
     b = oracle.attn_bwd_f64(bits(q), bits(k), bits(v), bits(g), True, 0.3)
     for x, y in zip(a, b):
         np.testing.assert_allclose(x, y, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_bwd_ex_arbitrary_key_mask_matches_autograd_of_the_libtorch_padding_mask(causal):
+    from oracle import libtorch_path as lt
+    B, Hq, Hkv, N, D = 2, 4, 2, 40, 16
+    q, g = lt.make_inputs(71, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(72, (B, Hkv, N, D), (B, Hkv, N, D))
+    gen = torch.Generator().manual_seed(73)
+    km = torch.rand(B, N, generator=gen) < 0.6
+    km[:, 0] = True
+    dq, dk, dv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), causal, 0.25, key_mask=km.numpy())
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    # lean_torch_sdpa_gqa_mask scales by 1/sqrt(D) = 0.25 at D = 16
+    out = lt.sdpa_gqa_mask(q64, k64, v64, km.long(), causal)
+    out.backward(g.double())
+    np.testing.assert_allclose(dq, q64.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dk, k64.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dv, v64.grad.numpy(), rtol=1e-4, atol=1e-5)
+    # hidden keys get no gradient
+    hidden = ~km.unsqueeze(1).expand(B, Hkv, N)
+    assert np.all(dk[hidden.numpy()] == 0) and np.all(dv[hidden.numpy()] == 0)

@@ -12,7 +12,7 @@ LIB_PATH = os.environ.get("TYR_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libt
 SYMBOLS = (
     "tyr_hip_strerror", "tyr_hip_version", "tyr_hip_device_info", "tyr_hip_check_device_pointer",
     "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_fwd_gqa", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
-    "tyr_hip_flash_attn_bwd_gqa",
+    "tyr_hip_flash_attn_bwd_gqa", "tyr_hip_flash_attn_fwd_mask", "tyr_hip_flash_attn_bwd_mask",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
     "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
     "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy",
@@ -51,6 +51,10 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_flash_attn_bwd.restype = ci
     L.tyr_hip_flash_attn_bwd_gqa.argtypes = [vp] * 9 + [u64] * 5 + [ci, u64, vp, f32, vp, sz, vp]
     L.tyr_hip_flash_attn_bwd_gqa.restype = ci
+    L.tyr_hip_flash_attn_fwd_mask.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, u64, ci, vp, f32, vp]
+    L.tyr_hip_flash_attn_fwd_mask.restype = ci
+    L.tyr_hip_flash_attn_bwd_mask.argtypes = [vp] * 9 + [u64] * 5 + [ci, vp, f32, vp, sz, vp]
+    L.tyr_hip_flash_attn_bwd_mask.restype = ci
     L.tyr_hip_gqa_decode_workspace_bytes.argtypes = [u64] * 6
     L.tyr_hip_gqa_decode_workspace_bytes.restype = sz
     L.tyr_hip_gqa_decode_auto_splits.argtypes = [u64] * 3

@@ -91,10 +91,10 @@ int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
     return tyr_hip_flash_attn_fwd_gqa(q, k, v, o, lse, B, H, H, N, D, causal, 0, nullptr, scale, stream);
 }
 
-int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void* o, float* lse,
-                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
-                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
-                               void* stream) {
+static int attn_fwd_checked(const void* q, const void* k, const void* v, void* o, float* lse,
+                            uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                            int causal, uint64_t window, const int32_t* kv_lens, const uint8_t* key_mask,
+                            float scale, void* stream) {
     if (!q || !k || !v || !o) return TYR_HIP_ERR_NULL_POINTER;
     if (B == 0 || Hq == 0 || Hkv == 0 || N == 0 || D == 0 || Hq % Hkv != 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return TYR_HIP_ERR_UNSUPPORTED;
@@ -108,8 +108,22 @@ int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void
     if (kv_lens && (reinterpret_cast<uintptr_t>(kv_lens) & 3u)) return TYR_HIP_ERR_MISALIGNED;
     const int rc = tyr::launch_flash_attn_fwd(q, k, v, o, lse, (int)B, (int)Hq, (int)Hkv, (int)N, (int)D,
                                               causal != 0, (int)(window > (uint64_t)INT_MAX ? INT_MAX : window),
-                                              kv_lens, scale, static_cast<hipStream_t>(stream));
+                                              kv_lens, key_mask, scale, static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void* o, float* lse,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* stream) {
+    return attn_fwd_checked(q, k, v, o, lse, B, Hq, Hkv, N, D, causal, window, kv_lens, nullptr, scale, stream);
+}
+
+int tyr_hip_flash_attn_fwd_mask(const void* q, const void* k, const void* v, void* o, float* lse,
+                                uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                int causal, const uint8_t* key_mask, float scale, void* stream) {
+    if (!key_mask) return TYR_HIP_ERR_NULL_POINTER;
+    return attn_fwd_checked(q, k, v, o, lse, B, Hq, Hkv, N, D, causal, 0, nullptr, key_mask, scale, stream);
 }
 
 size_t tyr_hip_flash_attn_bwd_workspace_bytes(uint64_t B, uint64_t H, uint64_t N, uint64_t D) {
@@ -126,11 +140,11 @@ int tyr_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const vo
                                       workspace, workspace_bytes, stream);
 }
 
-int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, const void* o,
-                               const void* d_o, const float* lse, void* dq, void* dk, void* dv,
-                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
-                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
-                               void* workspace, size_t workspace_bytes, void* stream) {
+static int attn_bwd_checked(const void* q, const void* k, const void* v, const void* o,
+                            const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                            uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                            int causal, uint64_t window, const int32_t* kv_lens, const uint8_t* key_mask,
+                            float scale, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return TYR_HIP_ERR_NULL_POINTER;
     if (B == 0 || Hq == 0 || Hkv == 0 || N == 0 || D == 0 || Hq % Hkv != 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return TYR_HIP_ERR_UNSUPPORTED;
@@ -150,9 +164,28 @@ int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, cons
     if (!aligned16(workspace)) return TYR_HIP_ERR_MISALIGNED;
     const int rc = tyr::launch_flash_attn_bwd(q, k, v, o, d_o, lse, dq, dk, dv, (int)B, (int)Hq, (int)Hkv, (int)N,
                                               (int)D, causal != 0,
-                                              (int)(window > (uint64_t)INT_MAX ? INT_MAX : window), kv_lens, scale,
-                                              workspace, static_cast<hipStream_t>(stream));
+                                              (int)(window > (uint64_t)INT_MAX ? INT_MAX : window), kv_lens, key_mask,
+                                              scale, workspace, static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_flash_attn_bwd_gqa(const void* q, const void* k, const void* v, const void* o,
+                               const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                               uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                               int causal, uint64_t window, const int32_t* kv_lens, float scale,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_bwd_checked(q, k, v, o, d_o, lse, dq, dk, dv, B, Hq, Hkv, N, D, causal, window, kv_lens, nullptr,
+                            scale, workspace, workspace_bytes, stream);
+}
+
+int tyr_hip_flash_attn_bwd_mask(const void* q, const void* k, const void* v, const void* o,
+                                const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                                uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                int causal, const uint8_t* key_mask, float scale,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+    if (!key_mask) return TYR_HIP_ERR_NULL_POINTER;
+    return attn_bwd_checked(q, k, v, o, d_o, lse, dq, dk, dv, B, Hq, Hkv, N, D, causal, 0, nullptr, key_mask,
+                            scale, workspace, workspace_bytes, stream);
 }
 
 uint64_t tyr_hip_gqa_decode_auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {

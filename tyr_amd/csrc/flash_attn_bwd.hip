@@ -125,7 +125,8 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     const uint16_t* __restrict__ O, const uint16_t* __restrict__ dO, const float* __restrict__ LSE,
     uint16_t* __restrict__ dQ, float2* __restrict__ stats, int BH, int N, int ntq, float scale,
-    float scale_log2, int Hq, int G, int window, const int* __restrict__ kv_lens, int pair) {
+    float scale_log2, int Hq, int G, int window, const int* __restrict__ kv_lens,
+    const uint8_t* __restrict__ key_mask, int pair) {
     using namespace fab;
     using C = CfgQ<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -164,6 +165,7 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const uint16_t* Kh = Kp + (size_t)kvbh * N * D;
     const uint16_t* Vh = Vp + (size_t)kvbh * N * D;
     const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    const uint8_t* km = (EXT && key_mask != nullptr) ? key_mask + (size_t)(bh / Hq) * N : nullptr;
     const int kv_end = CAUSAL ? min(Nk, q0 + C::BM) : Nk;
     const int nkv_abs = (kv_end + C::BN - 1) / C::BN;
     const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / C::BN, nkv_abs - 1) : 0;
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             f32x16 s[2], dp[2];
             bf16x8 dsf[4];
             const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
-                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && km != nullptr);
             auto scores = [&](int T) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
@@ -279,10 +281,19 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
                     const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;
                     const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;
                     const int base = j0 + 4 * g;
+                    uint32_t hidden = 0;             // bit e: the key mask hides this lane's kv row
+                    if (EXT && km != nullptr) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
+                            hidden |= (km[min(kv, N - 1)] == 0 ? 1u : 0u) << e;
+                        }
+                    }
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        if (kv > lim || (EXT && kv < low)) s[T][e] = -INFINITY;
+                        const bool off = kv > lim || (EXT && kv < low) || ((hidden >> e) & 1u);
+                        s[T][e] = off ? -INFINITY : s[T][e];
                     }
                 }
 #pragma unroll
@@ -338,7 +349,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     const uint16_t* __restrict__ dO, const float2* __restrict__ stats, uint16_t* __restrict__ dK,
     uint16_t* __restrict__ dV, int BHkv, int N, int ntk, int npad, float scale, float scale_log2,
-    int Hq, int G, int window, const int* __restrict__ kv_lens) {
+    int Hq, int G, int window, const int* __restrict__ kv_lens, const uint8_t* __restrict__ key_mask) {
     using namespace fab;
     using C = CfgK<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -366,6 +377,8 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const int hkv = Hq / G;
     const size_t qh0 = (size_t)(bh / hkv) * Hq + (size_t)(bh % hkv) * G;   // first query head of the group
     const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / hkv])) : N;
+    // this lane's key is hidden from every query by the key mask
+    const bool key_off = EXT && key_mask != nullptr && key_mask[(size_t)(bh / hkv) * N + min(kvpos, N - 1)] == 0;
 
     // ---- this wave's K and V rows as column operands (lane = key row, columns 16i + 8g + [0,8))
     bf16x8 kf[C::KSTEPS], vf[C::KSTEPS];
@@ -524,7 +537,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
                     for (int x = 0; x < 4; ++x) {
                         const int qrow = qs0 + 8 * (2 * sh + h) + 4 * g + x;
                         const bool hidden = (CAUSAL && kvpos > qrow) ||
-                                            (EXT && ((window > 0 && qrow - kvpos >= window) || kvpos >= Nk));
+                                            (EXT && ((window > 0 && qrow - kvpos >= window) || kvpos >= Nk || key_off));
                         if (hidden) p[x] = 0.0f;
                     }
                 }
@@ -678,13 +691,14 @@ size_t flash_attn_bwd_workspace_bytes(int B, int H, int N) {
 
 int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                           const float* lse, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int N, int D,
-                          int causal, int window, const int* kv_lens, float scale, void* workspace,
+                          int causal, int window, const int* kv_lens, const uint8_t* key_mask, float scale,
+                          void* workspace,
                           hipStream_t stream) {
     using namespace fab;
     const int BH = B * Hq, BHkv = B * Hkv, G = Hq / Hkv;
     const int ntq = (N + 127) / 128;
     const int npad = ntq * 128;
-    const bool ext = window > 0 || kv_lens != nullptr;
+    const bool ext = window > 0 || kv_lens != nullptr || key_mask != nullptr;
     const int pair = (causal && !ext && ntq > 1) ? 1 : 0;
     dim3 grid_q((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), grid_k((unsigned)(BHkv * ntq)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
@@ -705,11 +719,11 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
         if (a1 != hipSuccess || a2 != hipSuccess) return -1;                                          \
         hipLaunchKernelGGL((flash_attn_bwd_dq_kernel<DD, CC, EE>), grid_q, block, CfgQ<DD>::LDS, stream, \
                            Qp, Kp, Vp, Op, dOp, lse, static_cast<uint16_t*>(dq), st, BH, N, ntq,      \
-                           scale, scale_log2, Hq, G, window, kv_lens, pair);                          \
+                           scale, scale_log2, Hq, G, window, kv_lens, key_mask, pair);                \
         hipLaunchKernelGGL((flash_attn_bwd_dkv_kernel<DD, CC, EE>), grid_k, block, CfgK<DD>::LDS, stream, \
                            Qp, Kp, Vp, dOp, st, static_cast<uint16_t*>(dk),                           \
                            static_cast<uint16_t*>(dv), BHkv, N, ntq, npad, scale, scale_log2, Hq, G,  \
-                           window, kv_lens);                                                          \
+                           window, kv_lens, key_mask);                                                \
     } while (0)
 #define TYR_FAB_PICK(DD)                                                                              \
     do {                                                                                              \

@@ -71,7 +71,7 @@ template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2,
-    int Hq, int G, int window, const int* __restrict__ kv_lens, int pair) {
+    int Hq, int G, int window, const int* __restrict__ kv_lens, const uint8_t* __restrict__ key_mask, int pair) {
     using namespace fa;
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -121,6 +121,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
     // keys at or beyond Nk are masked; with a window, query i sees keys (i - window, i]
     const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    // per-sequence key mask (nonzero = visible), any pattern
+    const uint8_t* km = (EXT && key_mask != nullptr) ? key_mask + (size_t)(bh / Hq) * N : nullptr;
     const int kv_end = CAUSAL ? min(Nk, q0 + BM) : Nk;
     const int nkv_abs = (kv_end + BN - 1) / BN;
     const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / BN, nkv_abs - 1) : 0;   // first tile any row sees
@@ -260,17 +262,30 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             // ---- mask (diagonal tiles, ragged tail) -- register e of sub-tile T is kv row
             //      j0 + 32T + 8(e/4) + 4g + e%4
             const bool need_mask = (CAUSAL && (j0 + BN - 1 > qw0)) || (j0 + BN > Nk) ||
-                                   (EXT && window > 0 && j0 < qw0 + 32 - window);
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && km != nullptr);
             if (need_mask) {
                 const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;   // largest visible kv row
                 const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;   // smallest visible kv row
                 const int base = j0 + 4 * g;
+                // bit 16T+e: the key mask hides this lane's kv row (gathered first, so that the
+                // masking below is one select per score)
+                uint32_t hidden = 0;
+                if (EXT && km != nullptr) {
+#pragma unroll
+                    for (int T = 0; T < 2; ++T)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
+                            hidden |= (km[min(kv, N - 1)] == 0 ? 1u : 0u) << (16 * T + e);
+                        }
+                }
 #pragma unroll
                 for (int T = 0; T < 2; ++T)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        if (kv > lim || (EXT && kv < low)) cur[T][e] = -INFINITY;
+                        const bool off = kv > lim || (EXT && kv < low) || ((hidden >> (16 * T + e)) & 1u);
+                        cur[T][e] = off ? -INFINITY : cur[T][e];
                     }
             }
 
@@ -398,12 +413,13 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                           int Hq, int Hkv, int N, int D, int causal, int window, const int* kv_lens,
+                          const uint8_t* key_mask,
                           float scale, hipStream_t stream) {
     using namespace fa;
     const int BH = B * Hq;
     const int G = Hq / Hkv;
     const int ntq = (N + BM - 1) / BM;
-    const bool ext = window > 0 || kv_lens != nullptr;
+    const bool ext = window > 0 || kv_lens != nullptr || key_mask != nullptr;
     const int pair = (causal && !ext && ntq > 1) ? 1 : 0;
     dim3 grid((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), block(THREADS);
     const float scale_log2 = scale * LOG2E;
@@ -418,7 +434,7 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DD>::LDS);                           \
         if (attr != hipSuccess) return -1;                                                       \
         hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC, EE>), grid, block, Cfg<DD>::LDS, stream, \
-                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens, pair); \
+                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens, key_mask, pair); \
     } while (0)
 #define TYR_FA_PICK(DD)                                                                          \
     do {                                                                                         \

@@ -13,12 +13,12 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
                     int trans_b, hipStream_t stream);
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                           int Hq, int Hkv, int N, int D, int causal, int window, const int* kv_lens,
-                          float scale, hipStream_t stream);
+                          const uint8_t* key_mask, float scale, hipStream_t stream);
 size_t flash_attn_bwd_workspace_bytes(int B, int H, int N);
 int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                           const float* lse, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int N, int D,
-                          int causal, int window, const int* kv_lens, float scale, void* workspace,
-                          hipStream_t stream);
+                          int causal, int window, const int* kv_lens, const uint8_t* key_mask, float scale,
+                          void* workspace, hipStream_t stream);
 int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                       int Hq, int Hkv, int L, int D, int64_t kv_stride, float scale, int num_splits,
                       void* workspace, const int* kv_lens, int window, hipStream_t stream);

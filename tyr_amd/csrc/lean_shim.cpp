@@ -183,6 +183,69 @@ lean_object* lean_tyr_gpu_flash_attn_bwd_gqa(uint64_t B, uint64_t Hq, uint64_t H
     }
 }
 
+// flashAttnFwdMask {B Hq Hkv N D} q k v keyMask causal scale stream : IO (T #[B,Hq,N,D] x T #[B,Hq,N])
+// keyMask : uint8 [B, N], nonzero = visible key (the mask argument of lean_torch_sdpa_gqa_mask as bytes)
+lean_object* lean_tyr_gpu_flash_attn_fwd_mask(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                              b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                              b_lean_obj_arg key_mask, uint8_t causal, double scale,
+                                              uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v), m_ = borrowTensor(key_mask);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err) || !check(m_, "keyMask", torch::kUInt8, err))
+            return io_error(err);
+        if ((uint64_t)m_.numel() != B * N) return io_error("flashAttnFwdMask: keyMask must hold B*N bytes");
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)Hq, (int64_t)N}, q_.options().dtype(torch::kFloat32));
+        const int rc = tyr_hip_flash_attn_fwd_mask(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                                   lse.data_ptr<float>(), B, Hq, Hkv, N, D, causal,
+                                                   m_.data_ptr<uint8_t>(), (float)scale,
+                                                   reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnFwdMask", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// flashAttnBwdMask {B Hq Hkv N D} q k v o lse dO keyMask causal scale stream : IO (dQ x dK x dV)
+lean_object* lean_tyr_gpu_flash_attn_bwd_mask(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                              b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                              b_lean_obj_arg o, b_lean_obj_arg lse, b_lean_obj_arg d_o,
+                                              b_lean_obj_arg key_mask, uint8_t causal, double scale,
+                                              uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v), o_ = borrowTensor(o);
+        auto lse_ = borrowTensor(lse), g_ = borrowTensor(d_o), m_ = borrowTensor(key_mask);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err) || !check(o_, "o", torch::kBFloat16, err) ||
+            !check(g_, "dO", torch::kBFloat16, err) || !check(lse_, "lse", torch::kFloat32, err) ||
+            !check(m_, "keyMask", torch::kUInt8, err))
+            return io_error(err);
+        if ((uint64_t)m_.numel() != B * N) return io_error("flashAttnBwdMask: keyMask must hold B*N bytes");
+        auto dq = torch::empty_like(q_), dk = torch::empty_like(k_), dv = torch::empty_like(k_);
+        const size_t ws_bytes = tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D);
+        auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
+        const int rc = tyr_hip_flash_attn_bwd_mask(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o_.data_ptr(),
+                                                   g_.data_ptr(), lse_.data_ptr<float>(), dq.data_ptr(),
+                                                   dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, N, D, causal,
+                                                   m_.data_ptr<uint8_t>(), (float)scale, ws.data_ptr(), ws_bytes,
+                                                   reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnBwdMask", rc);
+        lean_object* inner = lean_alloc_ctor(0, 2, 0);
+        lean_ctor_set(inner, 0, giveTensor(std::move(dk)));
+        lean_ctor_set(inner, 1, giveTensor(std::move(dv)));
+        lean_object* outer = lean_alloc_ctor(0, 2, 0);
+        lean_ctor_set(outer, 0, giveTensor(std::move(dq)));
+        lean_ctor_set(outer, 1, inner);
+        return lean_io_result_mk_ok(outer);
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 // gqaDecode {B Hq Hkv L D} q k v scale numSplits stream : IO (T #[B,Hq,1,D] x T #[B,Hq])
 lean_object* lean_tyr_gpu_gqa_decode(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
                                      b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v, double scale,

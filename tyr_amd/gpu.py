@@ -67,13 +67,28 @@ def device_info(device: int = 0) -> dict:
             "clock_mhz": clk.value, "hbm_bytes": hbm.value}
 
 
+def _key_mask_ptr(key_mask, B, N, window, kv_lens):
+    """Device pointer of a [B, N] key mask (bool or uint8, nonzero = visible)."""
+    if window or kv_lens is not None:
+        raise TyrGpuError("a key mask cannot be combined with a window or key lengths")
+    if not isinstance(key_mask, torch.Tensor):
+        raise TyrGpuError("keyMask must be a tensor")
+    if key_mask.dtype not in (torch.bool, torch.uint8):
+        raise TyrGpuError("keyMask must have dtype torch.bool or torch.uint8")
+    _check(key_mask, "keyMask", key_mask.dtype, 2)
+    if tuple(key_mask.shape) != (B, N):
+        raise TyrGpuError("keyMask must have shape [B, N]")
+    return key_mask.data_ptr()
+
+
 def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, window: int = 0, kv_lens=None,
-                   stream=None):
+                   key_mask=None, stream=None):
     """O, LSE = flashAttnFwd q k v causal scale.
 
     q bf16 [B,Hq,N,D]; k, v bf16 [B,Hkv,N,D] with Hq % Hkv == 0 (query head h reads kv head h / (Hq/Hkv));
     ``window`` > 0 (causal only) lets query i see keys (i - window, i]; ``kv_lens`` (int32 [B] on the device)
-    masks the keys at or beyond each sequence's length.  -> (bf16 [B,Hq,N,D], f32 [B,Hq,N])."""
+    masks the keys at or beyond each sequence's length; ``key_mask`` (bool / uint8 [B,N] on the device, nonzero =
+    visible) hides any set of keys per sequence instead.  -> (bf16 [B,Hq,N,D], f32 [B,Hq,N])."""
     for t, n in ((q, "q"), (k, "k"), (v, "v")):
         _check(t, n, torch.bfloat16, 4)
     B, Hq, N, D = q.shape
@@ -92,6 +107,13 @@ def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, win
         lens_ptr = kv_lens.data_ptr()
     o = torch.empty_like(q)
     lse = torch.empty((B, Hq, N), dtype=torch.float32, device=q.device)
+    if key_mask is not None:
+        rc = _lib.load().tyr_hip_flash_attn_fwd_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                     lse.data_ptr(), B, Hq, Hkv, N, D, int(bool(causal)),
+                                                     _key_mask_ptr(key_mask, B, N, window, kv_lens), float(scale),
+                                                     _stream(stream))
+        _raise(rc, "flashAttnFwd")
+        return o, lse
     rc = _lib.load().tyr_hip_flash_attn_fwd_gqa(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                                 lse.data_ptr(), B, Hq, Hkv, N, D, int(bool(causal)), int(window),
                                                 lens_ptr, float(scale), _stream(stream))
@@ -100,11 +122,11 @@ def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, win
 
 
 def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | None = None, window: int = 0,
-                   kv_lens=None, stream=None):
+                   kv_lens=None, key_mask=None, stream=None):
     """dQ, dK, dV = flashAttnBwd q k v o lse dO causal scale.
 
     q, o, d_o bf16 [B,Hq,N,D]; k, v bf16 [B,Hkv,N,D]; lse f32 [B,Hq,N]; o and lse as returned by
-    flash_attn_fwd for the same q, k, v, causal, scale, window and kv_lens.  Returns dQ [B,Hq,N,D] and
+    flash_attn_fwd for the same q, k, v, causal, scale, window, kv_lens and key_mask.  Returns dQ [B,Hq,N,D] and
     dK, dV [B,Hkv,N,D] (summed over the query heads of each kv head), bf16."""
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "dO")):
         _check(t, n, torch.bfloat16, 4)
@@ -131,6 +153,13 @@ def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | Non
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(k)
     nbytes = lib.tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D)
     ws = torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=q.device)
+    if key_mask is not None:
+        rc = lib.tyr_hip_flash_attn_bwd_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
+                                             lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, N,
+                                             D, int(bool(causal)), _key_mask_ptr(key_mask, B, N, window, kv_lens),
+                                             float(scale), ws.data_ptr(), ws.numel(), _stream(stream))
+        _raise(rc, "flashAttnBwd")
+        return dq, dk, dv
     rc = lib.tyr_hip_flash_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
                                         lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, N, D,
                                         int(bool(causal)), int(window), lens_ptr, float(scale), ws.data_ptr(),

@@ -73,6 +73,23 @@ opaque flashAttnBwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : 
     (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
     : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
 
+/-- `flashAttnFwdGQA` with an arbitrary key mask instead of lengths: `keyMask : uint8 [B,N]`, key `j` of
+    sequence `b` is visible iff `keyMask[b,j] ≠ 0` (and `j ≤ i` when `causal`). GPU twin of
+    `nn.scaledDotProductAttentionGQAMask` (`cc/src/tyr.cpp:4019-4095`) for any mask, e.g. left padding;
+    a row that sees no key gets `O = 0`, `LSE = -∞` where LibTorch returns NaN. -/
+@[extern "lean_tyr_gpu_flash_attn_fwd_mask"]
+opaque flashAttnFwdMask {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (keyMask : @& T #[B, N]) (causal : Bool) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hq, N])
+
+/-- Backward of `flashAttnFwdMask` (same `q k v keyMask causal scale`; `o lse` its results): hidden keys
+    receive `dK = dV = 0`, rows that saw no key `dQ = 0`. -/
+@[extern "lean_tyr_gpu_flash_attn_bwd_mask"]
+opaque flashAttnBwdMask {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (o : @& T #[B, Hq, N, D]) (lse : @& T #[B, Hq, N]) (dO : @& T #[B, Hq, N, D]) (keyMask : @& T #[B, N])
+    (causal : Bool) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
+
 /-- GQA decode attention, one query token per sequence, split-KV with an LSE combine pass.
     `q : bf16 [B,Hq,1,D]`, `k v : bf16 [B,Hkv,L,D]` (contiguous cache), `D ∈ {64, 128}`,
     query head `h` reads kv head `h / (Hq/Hkv)`; `numSplits = 0` lets the library choose.
