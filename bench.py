@@ -58,6 +58,16 @@ def _events(torch, n):
 # goes from 128 to 111 us per launch over its first 15 ms).  Every workload therefore runs untimed for
 # this long before its W warm-up steps; the timed region is still exactly K steps.
 PREWARM_MS = 80.0
+# "randn" is the benchmark input.  "constant" fills every operand with 0.5: the same instruction stream
+# with almost no bit toggling, which shows how much of the time is the device holding its clock down
+# under the power the data draws (a diagnostic, never a headline number).
+DATA = "randn"
+
+
+def _normal(torch, *shape):
+    if DATA == "constant":
+        return torch.full(shape, 0.5, device="cuda")
+    return torch.randn(*shape, device="cuda")
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -86,7 +96,7 @@ def time_steps(torch, fn, steps, warmup):
 def wl_attn(torch, tyr, steps, warmup, cpu):
     B, H, N, D = 16, 16, 4096, 128
     torch.manual_seed(0)
-    q, k, v = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(3))
+    q, k, v = (_normal(torch, B, H, N, D).to(torch.bfloat16) for _ in range(3))
     sc = 1.0 / math.sqrt(D)
     fn = lambda: tyr.flash_attn_fwd(q, k, v, causal=True, scale=sc)
     wall, ms = time_steps(torch, fn, steps, warmup)
@@ -121,7 +131,7 @@ def wl_attn(torch, tyr, steps, warmup, cpu):
 def wl_attn_bwd(torch, tyr, steps, warmup, cpu):
     B, H, N, D = 16, 16, 4096, 128
     torch.manual_seed(0)
-    q, k, v, g = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(4))
+    q, k, v, g = (_normal(torch, B, H, N, D).to(torch.bfloat16) for _ in range(4))
     sc = 1.0 / math.sqrt(D)
     o, lse = tyr.flash_attn_fwd(q, k, v, causal=True, scale=sc)
     fn = lambda: tyr.flash_attn_bwd(q, k, v, o, lse, g, causal=True, scale=sc)
@@ -205,8 +215,8 @@ def wl_decode(torch, tyr, steps, warmup, cpu):
 def wl_gemm_bf16(torch, tyr, steps, warmup, cpu):
     M = N = K = 4096
     torch.manual_seed(2)
-    a = (torch.randn(M, K, device="cuda") * K ** -0.25).to(torch.bfloat16)
-    b = (torch.randn(K, N, device="cuda") * K ** -0.25).to(torch.bfloat16)
+    a = (_normal(torch, M, K) * K ** -0.25).to(torch.bfloat16)
+    b = (_normal(torch, K, N) * K ** -0.25).to(torch.bfloat16)
     fn = lambda: tyr.gemm_bf16(a, b)
     wall, ms = time_steps(torch, fn, steps, warmup)
     tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
@@ -411,8 +421,11 @@ def main() -> int:
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
     ap.add_argument("--settle-ms", type=float, default=PREWARM_MS,
                     help="untimed work before the warm-up steps of every workload, in milliseconds")
+    ap.add_argument("--data", default="randn", choices=["randn", "constant"],
+                    help="operand values of the attention and bf16 GEMM workloads; 'constant' is a power diagnostic")
     args = ap.parse_args()
     globals()["PREWARM_MS"] = args.settle_ms
+    globals()["DATA"] = args.data
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
         return 2
@@ -433,7 +446,8 @@ def main() -> int:
         "steps": args.steps, "warmup": args.warmup, "settle_ms_before_warmup": PREWARM_MS,
         "ms_per_step": round(head["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
-        "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
+        "data": "synthetic" if DATA == "randn" else "synthetic, every operand 0.5 (power diagnostic, not the benchmark input)",
+        "config": head["config"], "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"), "wall_ms_per_step": round(head["wall_ms_per_step"], 5),
         "device": info,
     }

@@ -507,50 +507,50 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     };
     // P and dS of a sub-tile as column operands.  Register e <-> query row qs0 + 8(e/4) + 4g + e%4;
     // its (lse2, delta) pair sits at pair index 32T + 8(e/4) + 4g + e%4 of the staged kilobyte.
-    auto read_pairs = [&](auto stg, auto sub, f32x4 (&st)[8]) {
+    // Half sh of the pairs of sub-tile T: registers 8sh .. 8sh+7, i.e. k = e/4 in {2sh, 2sh+1}
+    auto read_pairs = [&](auto stg, auto sub, auto half, f32x4 (&st)[4]) {
         TYR_STG(stg);
-        constexpr int T = decltype(sub)::value;
+        constexpr int T = decltype(sub)::value, SH = decltype(half)::value;
         lds_cptr St = statp[STG >> 1] + SOFF + 32 * T * 8;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {                    // k = e/4
-            st[2 * k] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * k * 8);
-            st[2 * k + 1] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * k * 8 + 16);
+        for (int h = 0; h < 2; ++h) {                    // k = 2 SH + h
+            st[2 * h] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * (2 * SH + h) * 8);
+            st[2 * h + 1] = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(St + 8 * (2 * SH + h) * 8 + 16);
         }
     };
-    auto probabilities = [&](auto masked, const f32x4 (&st)[8], int qs0, const f32x16& s, const f32x16& dp,
-                             bf16x8 (&pf)[2], bf16x8 (&dsf)[2]) {
+    // P and dS of half sh of a sub-tile (query rows qs0 + 16sh + 8h + 4g + x) as one k-step of column operands
+    auto probabilities = [&](auto masked, auto half, const f32x4 (&st)[4], int qs0, const f32x16& s, const f32x16& dp,
+                             bf16x8& pf, bf16x8& dsf) {
         constexpr bool need_mask = decltype(masked)::value;
+        constexpr int sh = decltype(half)::value;
+        u32x4 ppk, dpk;
 #pragma unroll
-        for (int sh = 0; sh < 2; ++sh) {
-            u32x4 ppk, dpk;
+        for (int h = 0; h < 2; ++h) {                    // e/4 = 2sh + h
+            const f32x4 a = st[2 * h];
+            const f32x4 b = st[2 * h + 1];
+            const float l2[4] = {a[0], a[2], b[0], b[2]};
+            const float dl[4] = {a[1], a[3], b[1], b[3]};
+            float p[4], ds[4];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {                // e/4 = 2sh + h
-                const f32x4 a = st[2 * (2 * sh + h)];
-                const f32x4 b = st[2 * (2 * sh + h) + 1];
-                const float l2[4] = {a[0], a[2], b[0], b[2]};
-                const float dl[4] = {a[1], a[3], b[1], b[3]};
-                float p[4], ds[4];
+            for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
+            if (need_mask) {
 #pragma unroll
-                for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
-                if (need_mask) {
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const int qrow = qs0 + 8 * (2 * sh + h) + 4 * g + x;
-                        const bool hidden = (CAUSAL && kvpos > qrow) ||
-                                            (EXT && ((window > 0 && qrow - kvpos >= window) || kvpos >= Nk || key_off));
-                        if (hidden) p[x] = 0.0f;
-                    }
+                for (int x = 0; x < 4; ++x) {
+                    const int qrow = qs0 + 8 * (2 * sh + h) + 4 * g + x;
+                    const bool hidden = (CAUSAL && kvpos > qrow) ||
+                                        (EXT && ((window > 0 && qrow - kvpos >= window) || kvpos >= Nk || key_off));
+                    if (hidden) p[x] = 0.0f;
                 }
-#pragma unroll
-                for (int x = 0; x < 4; ++x) ds[x] = p[x] * (dp[8 * sh + 4 * h + x] - dl[x]);
-                ppk[2 * h] = pack_bf16(p[0], p[1]);
-                ppk[2 * h + 1] = pack_bf16(p[2], p[3]);
-                dpk[2 * h] = pack_bf16(ds[0], ds[1]);
-                dpk[2 * h + 1] = pack_bf16(ds[2], ds[3]);
             }
-            pf[sh] = __builtin_bit_cast(bf16x8, ppk);
-            dsf[sh] = __builtin_bit_cast(bf16x8, dpk);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) ds[x] = p[x] * (dp[8 * sh + 4 * h + x] - dl[x]);
+            ppk[2 * h] = pack_bf16(p[0], p[1]);
+            ppk[2 * h + 1] = pack_bf16(p[2], p[3]);
+            dpk[2 * h] = pack_bf16(ds[0], ds[1]);
+            dpk[2 * h + 1] = pack_bf16(ds[2], ds[3]);
         }
+        pf = __builtin_bit_cast(bf16x8, ppk);
+        dsf = __builtin_bit_cast(bf16x8, dpk);
     };
     // Transposed fragments of k-step c = 2T + sh (query rows 16c + 8h + 4g + [0,4)) of dO and Q
     auto read_transposed = [&](auto stg, int c, bf16x8 (&dot)[C::DT], bf16x8 (&qt)[C::DT]) {
@@ -569,44 +569,84 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     };
 
     bf16x8 rq[C::KSTEPS], rd[C::KSTEPS];              // row fragments of the next sub-tile, read one step ahead
-    // One step of the software pipeline on sub-tile u = 2t + T, tile t in stage STG (scores in sc /
-    // dpc): the score products of sub-tile u+1 (row fragments already in rq / rd) are issued among
-    // the exponentials of u, the row fragments of u+2 are requested under the dV / dK products of u.
-    // With one wave per SIMD nothing else hides LDS latency and every instruction of the wave costs
-    // issue time, so fragments are requested a phase ahead and addresses cost no instructions.
+    bf16x8 pf0, dsf0;                                 // P, dS of the first half of the current sub-tile
+    f32x4 st1[4];                                     // pairs of its second half
+    using Half0 = std::integral_constant<int, 0>;
+    using Half1 = std::integral_constant<int, 1>;
+    // One step of the software pipeline on sub-tile u = 2t + T, tile t in stage STG (scores in sc / dpc).
+    // With one wave per SIMD a vector instruction overlaps with the matrix pipe only where it sits
+    // between two MFMAs of the wave's own stream, and the pipe idles through any stretch of vector
+    // work that is longer than the MFMA before it.  The step therefore has two phases of 16 MFMAs,
+    // each carrying half a sub-tile's exponentials:
+    //   A: S, dP of sub-tile u+1 (row fragments already in rq / rd)  beside  P, dS of the second half of u
+    //   B: dV, dK of u (both halves)                                  beside  P, dS of the first half of u+1
+    // so that P, dS of a sub-tile's first half are always computed one step ahead (pf0 / dsf0).
+    // The row fragments of u+2 and the pairs of u+1 are requested a phase before they are used.
     // Past the last sub-tile the "next" reads hit a stage without live data; their results are dropped.
     auto step = [&](auto masked, auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc, f32x16& sn, f32x16& dpn) {
         constexpr int STG = decltype(stg)::value, T = decltype(sub)::value;
+        using Stg1 = std::integral_constant<int, T == 0 ? STG : ((STG + 1) & 3)>;       // stage of u+1
+        using Sub1 = std::integral_constant<int, 1 - T>;
         using Stg2 = std::integral_constant<int, (STG + 1) & 3>;                        // stage of u+2
         bf16x8 dot0[C::DT], qt0[C::DT], dot1[C::DT], qt1[C::DT];
+        f32x4 st0[4];
         read_transposed(stg, 2 * T, dot0, qt0);
-        f32x4 st[8];
-        read_pairs(stg, sub, st);
-        scores(rq, rd, sn, dpn);
-        bf16x8 pf[2], dsf[2];
-        probabilities(masked, st, qs0, sc, dpc, pf, dsf);
+        read_pairs(Stg1{}, Sub1{}, Half0{}, st0);
         read_transposed(stg, 2 * T + 1, dot1, qt1);
+        scores(rq, rd, sn, dpn);
+        bf16x8 pf1, dsf1;
+        probabilities(masked, Half1{}, st1, qs0, sc, dpc, pf1, dsf1);
+        read_pairs(Stg1{}, Sub1{}, Half1{}, st1);          // ahead of the row fragments: LDS answers in order
         read_rows(Stg2{}, sub, rq, rd);
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
-            dv[dt] = mfma_32x32x16_bf16(dot0[dt], pf[0], dv[dt]);
-            dk[dt] = mfma_32x32x16_bf16(qt0[dt], dsf[0], dk[dt]);
+            dv[dt] = mfma_32x32x16_bf16(dot0[dt], pf0, dv[dt]);
+            dk[dt] = mfma_32x32x16_bf16(qt0[dt], dsf0, dk[dt]);
         }
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt) {
-            dv[dt] = mfma_32x32x16_bf16(dot1[dt], pf[1], dv[dt]);
-            dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf[1], dk[dt]);
+            dv[dt] = mfma_32x32x16_bf16(dot1[dt], pf1, dv[dt]);
+            dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf1, dk[dt]);
         }
+        probabilities(masked, Half0{}, st0, qs0 + 32, sn, dpn, pf0, dsf0);
+#ifndef TYR_DKV_NO_SCHED
+        // issue order: one MFMA, then its share of the LDS reads and of the vector work
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+        }
+#endif
     };
-    // What a step expects of the step before it, for the wave's first sub-tile: its scores, and the
-    // row fragments of the sub-tile after it.  Without EXT the only partially masked sub-tile of a
-    // causal wave is this one (its diagonal): hidden scores become -inf here, which the steps turn
-    // into P = 0 and dS = 0 like any other score, so they carry no mask instructions.
-    auto first_scores = [&](auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc) {
+    // What a step expects of the step before it, for the wave's first sub-tile: its scores, P and dS
+    // of its first half, the pairs of its second half, and the row fragments of the sub-tile after
+    // it.  Without EXT the only partially masked sub-tile of a causal wave is this one (its
+    // diagonal): hidden scores become -inf here, which the steps turn into P = 0 and dS = 0 like any
+    // other score, so they carry no mask instructions.
+    auto first_scores = [&](auto masked, auto stg, auto sub, int qs0, f32x16& sc, f32x16& dpc) {
         constexpr int STG = decltype(stg)::value, T = decltype(sub)::value;
         using Stg1 = std::integral_constant<int, T == 0 ? STG : ((STG + 1) & 3)>;     // stage of u+1
         using Sub1 = std::integral_constant<int, 1 - T>;
+        f32x4 st0[4];
         read_rows(stg, sub, rq, rd);
+        read_pairs(stg, sub, Half0{}, st0);
+        read_pairs(stg, sub, Half1{}, st1);
         scores(rq, rd, sc, dpc);
         if (CAUSAL && !EXT) {
 #pragma unroll
@@ -614,6 +654,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
                 if (kvpos > qs0 + 8 * (e >> 2) + 4 * g + (e & 3)) sc[e] = -INFINITY;
         }
         read_rows(Stg1{}, Sub1{}, rq, rd);
+        probabilities(masked, Half0{}, st0, qs0, sc, dpc, pf0, dsf0);
     };
 #undef TYR_STG
 
@@ -645,10 +686,10 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     if (u < nsub) {
         // u = u0 < 4: stage u0 / 2, sub-tile u0 % 2; even sub-tiles keep their scores in sA / dpA
         switch (u) {
-            case 0:  first_scores(integral_constant<int, 0>{}, integral_constant<int, 0>{}, qbase, sA, dpA); break;
-            case 1:  first_scores(integral_constant<int, 0>{}, integral_constant<int, 1>{}, qbase + 32, sB, dpB); break;
-            case 2:  first_scores(integral_constant<int, 1>{}, integral_constant<int, 0>{}, qbase + 64, sA, dpA); break;
-            default: first_scores(integral_constant<int, 1>{}, integral_constant<int, 1>{}, qbase + 96, sB, dpB); break;
+            case 0:  first_scores(MaskedT{}, integral_constant<int, 0>{}, integral_constant<int, 0>{}, qbase, sA, dpA); break;
+            case 1:  first_scores(MaskedT{}, integral_constant<int, 0>{}, integral_constant<int, 1>{}, qbase + 32, sB, dpB); break;
+            case 2:  first_scores(MaskedT{}, integral_constant<int, 1>{}, integral_constant<int, 0>{}, qbase + 64, sA, dpA); break;
+            default: first_scores(MaskedT{}, integral_constant<int, 1>{}, integral_constant<int, 1>{}, qbase + 96, sB, dpB); break;
         }
     }
     // the pipeline, unrolled over the 8 (stage, sub-tile) combinations; entered at u % 8
