@@ -42,7 +42,7 @@ PEAK = {"mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "hbm": 8000.0}   # TFLOP/s, TFL
 TRAFFIC = {"attn_fwd_causal": 1_073_162_240 + 272_629_760, "gqa_decode": 1_090_820_096 + 270_336,
            "gemm_bf16": 202_589_594 + 33_554_432, "gemm_fp8": 810_477_568 + 136_314_880,
            # both backward kernels: dQ (1,713,229,824 + 276,824,064) + dK/dV (1,082,617,856 + 536,870,912)
-           "attn_bwd_causal": 1_713_229_824 + 276_824_064 + 1_082_617_856 + 536_870_912,
+           "attn_bwd_causal": 1_647_249_408 + 276_824_064 + 1_082_636_288 + 536_870_912,
            "rope_kernel<bf16>": 270_592_000 + 268_437_504,
            "layernorm_residual_kernel<2>": 268_521_472 + 268_435_456,
            "copy_kernel": 1_073_784_832 + 1_073_848_320,
