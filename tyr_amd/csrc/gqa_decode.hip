@@ -9,8 +9,8 @@
 // partial results are merged with the online-softmax algebra
 //   m = max m_s ; l = sum l_s 2^(m_s-m) ; O = sum O_s 2^(m_s-m) / l ; LSE = ln l + m ln 2.
 //
-// First pass.  grid = (splits, B*Hkv), 8 waves per workgroup; each wave walks its own slice of
-// the split in steps of 32 kv rows with the 16x16x32 bf16 MFMA:
+// First pass.  grid = (splits, B*Hkv), 8 waves per workgroup; the waves take the 32-row steps of
+// the split in turn, each with the 16x16x32 bf16 MFMA:
 //   S^T (16 kv x 16 q)  = K rows (row operand: lane l holds row l%16, 8 d at 32i + 8(l/16))
 //                         x Q^T (column operand, zero beyond the G = Hq/Hkv real heads)
 //   O^T_j (16 d x 16 q) += V^T (row operand) x P^T (column operand),  j = 0..7
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     float* __restrict__ part_o, float* __restrict__ part_m, float* __restrict__ part_l,
     uint16_t* __restrict__ O, float* __restrict__ LSE,
-    int Hq, int Hkv, int G, int L, long kv_stride, int S, int chunk, int wchunk, float scale_log2,
+    int Hq, int Hkv, int G, int L, long kv_stride, int S, int chunk, float scale_log2,
     const int* __restrict__ kv_lens, int window) {
     using namespace dec;
     constexpr int THREADS = 64 * WAVES;
@@ -68,9 +68,12 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const int lo = window > 0 ? max(0, L - window) : 0;
     const int c0 = lo + split * chunk;
     const int c1 = min(L, c0 + chunk);
-    const int r0 = c0 + w * wchunk;             // this wave's rows [r0, r1)
-    const int r1 = min(c1, r0 + wchunk);
-    const int nsteps = r1 > r0 ? (r1 - r0 + STEP - 1) / STEP : 0;
+    // The waves of a workgroup take the 32-row steps of its chunk in turn (wave w: steps w, w + 8, ...),
+    // so the workgroup reads K and V as one contiguous front: +2 % over a contiguous slice per wave.
+    const int r0 = c0 + w * STEP;
+    const int r1 = c1;
+    constexpr int SST = WAVES * STEP;           // rows from one step of a wave to its next
+    const int nsteps = r1 > r0 ? (r1 - r0 + SST - 1) / SST : 0;
 
     // Q^T operand: column x = query head kvh*G + x (zero for x >= G)
     constexpr int KI = D / 32;                  // MFMA k-steps of a score tile
@@ -162,11 +165,11 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     Buf<D> b0, b1;
     if (nsteps > 0) load(b0, r0);
     for (int st = 0; st < nsteps; st += 2) {
-        if (st + 1 < nsteps) load(b1, r0 + (st + 1) * STEP);
-        compute(b0, r0 + st * STEP);
+        if (st + 1 < nsteps) load(b1, r0 + (st + 1) * SST);
+        compute(b0, r0 + st * SST);
         if (st + 1 < nsteps) {
-            if (st + 2 < nsteps) load(b0, r0 + (st + 2) * STEP);
-            compute(b1, r0 + (st + 1) * STEP);
+            if (st + 2 < nsteps) load(b0, r0 + (st + 2) * SST);
+            compute(b1, r0 + (st + 1) * SST);
         }
     }
 
@@ -250,8 +253,6 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
     const int span = window > 0 ? (window < L ? window : L) : L;     // longest range any sequence reads
     int chunk = (span + S - 1) / S;
     chunk = (chunk + STEP - 1) / STEP * STEP;
-    int wchunk = (chunk + WAVES - 1) / WAVES;
-    wchunk = (wchunk + STEP - 1) / STEP * STEP;
 
     float* part_o = static_cast<float*>(workspace);
     float* part_m = part_o + (size_t)B * Hq * S * D;
@@ -270,7 +271,7 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
                            static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k),         \
                            static_cast<const uint16_t*>(v), part_o, part_m, part_l,                  \
                            static_cast<uint16_t*>(o), lse, Hq, Hkv, G, L, (long)kv_stride, S, chunk, \
-                           wchunk, scale * LOG2E, kv_lens, window);                                  \
+                           scale * LOG2E, kv_lens, window);                                          \
         if (hipGetLastError() != hipSuccess) return -1;                                              \
         if (S > 1) {                                                                                 \
             hipLaunchKernelGGL(gqa_decode_combine_kernel<DD>, dim3((unsigned)(B * Hq)), dim3(DD), 0, \
