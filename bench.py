@@ -405,9 +405,31 @@ def wl_copy(torch, tyr, steps, warmup, cpu):
                          "unit": "GB/s", "frac": gbs / PEAK["hbm"], "traffic": 2.0 * n}}
 
 
+def wl_dsl_simple_gemm(torch, tyr, steps, warmup, cpu):
+    """The reference's example GEMM program (Tyr/GPU/Kernels/Examples.lean:23-65) emitted for gfx950 by
+    tyr_amd.dsl: one 64x64 tile per one-wave workgroup, single-buffered, as the program is written."""
+    from tyr_amd.dsl import kernels, runtime
+    M = N = 8192
+    K = 512
+    torch.manual_seed(0)
+    a = (_normal(torch, M, K) * K ** -0.25).to(torch.bfloat16)
+    b = (_normal(torch, K, N) * K ** -0.25).to(torch.bfloat16)
+    c = torch.zeros(M, N, device="cuda")
+    kern = kernels.simpleGemm()
+    fn = lambda: runtime.launch(kern, [a, b, c, M, N, K], grid=(N // 64, M // 64, 1), block=(32, 1, 1))   # one warp of the reference = one wave
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+    return {"metric": "emitted GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+            "dtype": "bf16",
+            "config": {"workload": "tile-DSL program simpleGemm emitted for gfx950, bf16 x bf16 -> f32, M=N=8192 K=512, "
+                                   "64x64 tile per one-wave workgroup"},
+            "roofline": {"bound": "mfma", "kernel": "simpleGemm (emitted)", "achieved": tf, "peak": PEAK["mfma_bf16"],
+                         "unit": "TFLOP/s", "frac": tf / PEAK["mfma_bf16"], "traffic": None}}
+
+
 WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "gqa_decode": wl_decode, "gemm_bf16": wl_gemm_bf16,
              "gemm_fp8": wl_gemm_fp8, "decode_step": wl_decode_step, "rope_fwd": wl_rope, "layernorm_residual": wl_layernorm,
-             "copy_kernel": wl_copy_kernel}
+             "copy_kernel": wl_copy_kernel, "dsl_simple_gemm": wl_dsl_simple_gemm}
 CALIBRATION = {"copy_1gib": wl_copy}
 
 
