@@ -479,7 +479,10 @@ def main() -> int:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
-            r = fn(torch, tyr_amd, max(10, args.steps // 2), max(3, args.warmup // 2), not args.no_cpu)
+            try:
+                r = fn(torch, tyr_amd, max(10, args.steps // 2), max(3, args.warmup // 2), not args.no_cpu)
+            except Exception as e:                      # a side workload must not take the headline line with it
+                r = {"error": f"{type(e).__name__}: {e}"}
             r["workload"] = name
             others.append(r)
         line["other_workloads"] = others
