@@ -221,3 +221,28 @@ def test_write_after_read_hazards_on_shared_tiles_get_barriers():
         k.store(s_, t)
     text = dsl.emit_kernel(k.build())
     assert text.index("// inserted:") < text.index("if (")
+
+
+def test_global_tiles_of_a_loop_are_requested_one_iteration_ahead():
+    # simpleGemm (Examples.lean:23-65) loads its A and B tiles at the top of the k loop: the emitter
+    # splits each load into the global read (into registers, issued for iteration i+1 after the first
+    # barrier of iteration i) and the write to LDS at the position of the original statement
+    src = dsl.emit_kernel(kernels.simpleGemm())
+    assert src.count("wave::gfrag<bf16, 64, 64>") == 2
+    assert src.count("wave::gload(") == 4 and src.count("wave::sstore(") == 2
+    loop = src[src.index("for (int"):]
+    assert loop.index("wave::sstore(") < loop.index("wave::sync();") < loop.index("wave::gload(") < loop.index("wave::mma_AB(")
+    plain = dsl.emit_kernel(kernels.simpleGemm(), prefetch_global_loads=False)
+    assert "gload" not in plain and plain.count("wave::load(") == 4
+    # a loop that also writes global memory keeps its loads where the program has them
+    k = dsl.KernelBuilder("copy_rows")
+    g, h = k.gptr("BFloat16", "src"), k.gptr("BFloat16", "dst")
+    c = k.blockCoord2D()
+    s_ = k.allocST("BFloat16", 64, 64)
+    with k.krange(0, 4) as i:
+        at = type(c)(c.b, c.d, i.id, c.c)
+        k.loadGlobal(s_, g, at)
+        k.sync()
+        k.storeGlobal(h, s_, at)
+        k.sync()
+    assert "gload" not in dsl.emit_kernel(k.build())

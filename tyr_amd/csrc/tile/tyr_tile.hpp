@@ -188,6 +188,33 @@ __device__ __forceinline__ void load(st<T, R, C>& dst, const gl<T>& src, coord a
     }
     wave_fence();
 }
+// The two halves of load(st, gl, at) with the pieces a lane moves held in registers in between:
+// the emitter requests the next iteration's tile of a loop before the products of the current one.
+template <typename T, int R, int C>
+struct gfrag {
+    static constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC, N = R * CPR / 64;
+    static_assert(C % VEC == 0 && (R * CPR) % 64 == 0, "tile is not a whole number of 16-byte pieces per lane");
+    u32x4 v[N];
+};
+template <typename T, int R, int C>
+__device__ __forceinline__ void gload(gfrag<T, R, C>& dst, const gl<T>& src, coord at) {
+    typedef gfrag<T, R, C> F;
+#pragma unroll
+    for (int k = 0; k < F::N; ++k) {
+        const int idx = lane() + 64 * k, r = idx / F::CPR, c = (idx % F::CPR) * F::VEC;
+        dst.v[k] = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
+    }
+}
+template <typename T, int R, int C>
+__device__ __forceinline__ void sstore(st<T, R, C>& dst, const gfrag<T, R, C>& src) {
+    typedef gfrag<T, R, C> F;
+#pragma unroll
+    for (int k = 0; k < F::N; ++k) {
+        const int idx = lane() + 64 * k, r = idx / F::CPR, c = (idx % F::CPR) * F::VEC;
+        *reinterpret_cast<u32x4*>(dst.at(r, c)) = src.v[k];
+    }
+    wave_fence();
+}
 template <typename T, int R, int C>
 __device__ __forceinline__ void store(const gl<T>& dst, const st<T, R, C>& src, coord at) {
     constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;

@@ -178,8 +178,11 @@ def shared_hazard_barriers(kernel: Kernel) -> set:
 
 
 class _Emitter:
-    def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True):
+    def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True,
+                 prefetch_global_loads: bool = True):
         self.k = kernel
+        # request the next iteration's global tiles of a loop before the work of the current one
+        self.prefetch_global_loads = prefetch_global_loads
         self.barrier_before = shared_hazard_barriers(kernel) if hazard_barriers else set()
         # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
         # full 512-register file, and covers the 128-thread blocks the reference's runners launch
@@ -306,12 +309,13 @@ class _Emitter:
             return f"{ind}wave::concat_cols({I(s.dst)}, {I(s.left)}, {I(s.right)});\n"
         if op == "sync":
             return f"{ind}wave::sync();\n"
-        if op == "forLoop":
-            return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < {s.hi}; ++{I(s.v)}) {{\n" + self.body(s.body, ind + "  ") +
+        if op in ("forLoop", "forLoopVal"):
+            hi = f"{s.hi}" if op == "forLoop" else f"(int){I(s.hi)}"
+            pre = self.prefetchable(s) if self.prefetch_global_loads else []
+            if pre:
+                return self.prefetched_loop(s, hi, pre, ind)
+            return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < {hi}; ++{I(s.v)}) {{\n" + self.body(s.body, ind + "  ") +
                     f"{ind}}}\n")
-        if op == "forLoopVal":
-            return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < (int){I(s.hi)}; ++{I(s.v)}) {{\n" +
-                    self.body(s.body, ind + "  ") + f"{ind}}}\n")
         if op == "ifStmt":
             out = f"{ind}if ({I(s.cond)}) {{\n" + self.body(s.thenBody, ind + "  ") + f"{ind}}}"
             if s.elseBody:
@@ -350,6 +354,72 @@ class _Emitter:
         if op == "raw":
             return f"{ind}{s.code}\n"
         raise UnsupportedStatement(op)
+
+    # ------------------------------------------------------------------ loops with prefetched tiles
+    def prefetchable(self, loop: Stmt):
+        """The leading loadGlobal statements of a loop body whose source and coordinates are the loop
+        variable or values defined outside the loop.  Their global reads can be issued one iteration
+        ahead (into registers) when nothing in the loop writes global memory."""
+        inner = list(walk(loop.body))
+        if any(t.op.startswith("store") and "Global" in t.op for t in inner):
+            return []
+        defined = {loop.v}
+        for t in inner:
+            for f in ("dst", "v"):
+                x = getattr(t, f, None)
+                if isinstance(x, VarId):
+                    defined.add(x)
+        out = []
+        for t in loop.body:
+            if t.op == "comment":
+                continue
+            if t.op != "loadGlobal" or id(t) in self.barrier_before:
+                break
+            free = all(c == loop.v or c not in defined for c in (t.coordB, t.coordD, t.coordR, t.coordC))
+            if not free or t.src in defined:
+                break
+            out.append(t)
+        # a tile loaded twice in the body, or written by another statement, keeps the plain form
+        written = [getattr(t, "dst", None) for t in inner if t not in out]
+        return [t for t in out if t.dst not in written and sum(1 for u in out if u.dst == t.dst) == 1]
+
+    def prefetched_loop(self, loop: Stmt, hi: str, pre, ind: str) -> str:
+        I = lambda v: v.ident
+        frag = {id(t): f"{I(t.dst)}_next" for t in pre}
+
+        def request(t, ind2):
+            tile = self.info[t.dst]
+            at = (f"coord{{(int){I(t.coordB)}, (int){I(t.coordD)}, (int){I(t.coordR)} * {tile.rows}, "
+                  f"(int){I(t.coordC)} * {tile.cols}}}")
+            return f"{ind2}wave::gload({frag[id(t)]}, {I(t.src)}, {at});\n"
+
+        out = f"{ind}// the global tiles of iteration i+1 are requested while iteration i computes\n"
+        for t in pre:
+            tile = self.info[t.dst]
+            out += f"{ind}wave::gfrag<{_cpp_type(tile.dtype)}, {tile.rows}, {tile.cols}> {frag[id(t)]};\n"
+        out += f"{ind}if ({loop.lo} < {hi}) {{\n{ind}  const int {I(loop.v)} = {loop.lo};\n"
+        out += "".join(request(t, ind + "  ") for t in pre) + f"{ind}}}\n"
+        out += f"{ind}for (int {I(loop.v)} = {loop.lo}; {I(loop.v)} < {hi}; ++{I(loop.v)}) {{\n"
+        ind2 = ind + "  "
+        nxt = (f"{ind2}if ({I(loop.v)} + 1 < {hi}) {{\n{ind2}  const int {I(loop.v)}_n = {I(loop.v)} + 1;\n"
+               f"{ind2}  {{\n{ind2}    const int {I(loop.v)} = {I(loop.v)}_n;\n" +
+               "".join(request(t, ind2 + "    ") for t in pre) + f"{ind2}  }}\n{ind2}}}\n")
+        placed = False
+        remaining = len(pre)
+        for t in loop.body:
+            if id(t) in self.barrier_before:
+                out += f"{ind2}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
+            if id(t) in frag:
+                out += f"{ind2}wave::sstore({I(t.dst)}, {frag[id(t)]});\n"
+                remaining -= 1
+                continue
+            out += self.stmt(t, ind2)
+            if not placed and remaining == 0 and t.op == "sync":
+                out += nxt
+                placed = True
+        if not placed:
+            out += nxt
+        return out + f"{ind}}}\n"
 
     def body(self, stmts, ind: str) -> str:
         out = ""
@@ -493,9 +563,9 @@ def emit_header(kernels: List[Kernel], cites: Dict[str, str]) -> str:
     return out + "#ifdef __cplusplus\n}\n#endif\n\n#endif /* TYR_DSL_KERNELS_H */\n"
 
 
-def emit_kernel(kernel: Kernel, hazard_barriers: bool = True) -> str:
+def emit_kernel(kernel: Kernel, hazard_barriers: bool = True, prefetch_global_loads: bool = True) -> str:
     """Device code of one kernel (no includes)."""
-    return _Emitter(kernel, hazard_barriers=hazard_barriers).kernel_text()
+    return _Emitter(kernel, hazard_barriers=hazard_barriers, prefetch_global_loads=prefetch_global_loads).kernel_text()
 
 
 def emit_translation_unit(kernels: List[Kernel]) -> str:
