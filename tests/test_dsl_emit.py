@@ -246,3 +246,28 @@ def test_global_tiles_of_a_loop_are_requested_one_iteration_ahead():
         k.storeGlobal(h, s_, at)
         k.sync()
     assert "gload" not in dsl.emit_kernel(k.build())
+
+
+def test_lds_tiles_with_disjoint_live_ranges_share_storage():
+    # simpleGemm: the f32 staging tile of the result is only used after the k loop, its A and B tiles
+    # only inside it -- one pool of 18,432 bytes instead of 35,840, i.e. twice the workgroups per CU
+    src = dsl.emit_kernel(kernels.simpleGemm())
+    assert "unsigned char tyr_lds_pool[18432];" in src
+    assert src.count("tyr_lds_pool + 0)") == 2 and "tyr_lds_pool + 9216)" in src
+    plain = dsl.emit_kernel(kernels.simpleGemm(), share_lds=False)
+    assert "tyr_lds_pool" not in plain and plain.count("__shared__ st<") == 3
+    # tiles that are live together never overlap: every pair of tiles used in one loop is disjoint
+    from tyr_amd.dsl.emit import lds_plan
+    for make in kernels.ALL:
+        k = make()
+        name = k.name
+        plan = lds_plan(k)
+        decl = {t.v: t for t in walk(k.body) if t.op == "declST"}
+        for body in [t.body for t in walk(k.body) if t.op in ("forLoop", "forLoopVal")]:
+            used = {a for t in walk(body) for a in t.args if isinstance(a, VarId) and a in plan}
+            spans = sorted((plan[v], plan[v] + decl[v].rows * decl[v].cols) for v in used)
+            assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), (name, spans)
+    # a kernel whose tiles are all live together keeps its plain declarations, and so does one where
+    # sharing would need a barrier the program does not have (the attention forward's Q and K tiles)
+    assert "tyr_lds_pool" not in dsl.emit_kernel(kernels.tkFusedLayerNormResidual1024())
+    assert "tyr_lds_pool" not in dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())

@@ -13,7 +13,7 @@ statements are no-ops because an MFMA is complete when its result is read.
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Any, Dict, List
 
 from .ir import GPU_FLOAT, K_SCALAR_TYPES, Kernel, Stmt, VarId, walk
 
@@ -111,7 +111,100 @@ def infer_rv_layouts(kernel: Kernel) -> Dict[VarId, str]:
     return out
 
 
-def shared_hazard_barriers(kernel: Kernel) -> set:
+_DTYPE_BYTES = {"Float32": 4, "BFloat16": 2, "Float16": 2, "FP8E4M3": 1, "FP8E5M2": 1}
+
+
+def _st_uses(s: Stmt, tiles) -> set:
+    """LDS tiles a (non-compound) statement touches."""
+    out = set()
+    for a in s.args:
+        if isinstance(a, VarId) and a in tiles:
+            out.add(a)
+    return out
+
+
+def lds_plan(kernel: Kernel) -> Dict[VarId, int]:
+    """Byte offsets of the LDS tiles in one pool, or {} when sharing storage saves nothing.
+
+    Tiles whose live ranges (first to last use in program order; a use inside a loop counts for the
+    whole loop) do not intersect may occupy the same bytes: a GEMM's output staging tile is only
+    used after the loop that uses its operand tiles.  Less LDS per workgroup is more workgroups per
+    CU."""
+    decl = {s.v: s for s in walk(kernel.body) if s.op == "declST"}
+    if len(decl) < 2:
+        return {}
+    size = {}
+    for v, d in decl.items():
+        b = _DTYPE_BYTES.get(d.dtype)
+        if b is None:
+            return {}
+        size[v] = (d.rows * (d.cols * b + 16) + 15) // 16 * 16
+    live: Dict[VarId, List[int]] = {}
+    pos = [0]
+
+    def touch(v, a, b):
+        r = live.setdefault(v, [a, b])
+        r[0], r[1] = min(r[0], a), max(r[1], b)
+
+    def run(body):
+        for s in body:
+            pos[0] += 1
+            if s.op in ("forLoop", "forLoopVal"):
+                start = pos[0]
+                before = {v: list(r) for v, r in live.items()}
+                run(s.body)
+                end = pos[0]
+                for v, r in live.items():
+                    if before.get(v) != r:               # used inside the loop: live for all of it
+                        touch(v, start, end)
+            elif s.op == "ifStmt":
+                run(s.thenBody)
+                run(s.elseBody)
+            elif s.op != "declST":
+                for v in _st_uses(s, decl):
+                    touch(v, pos[0], pos[0])
+
+    run(kernel.body)
+    placed: Dict[VarId, int] = {}
+    for v in sorted(decl, key=lambda t: -size[t]):
+        if v not in live:
+            live[v] = [0, 0]
+        off = 0
+        while True:
+            clash = [u for u in placed
+                     if not (live[u][1] < live[v][0] or live[v][1] < live[u][0])
+                     and off < placed[u] + size[u] and placed[u] < off + size[v]]
+            if not clash:
+                break
+            off = max(placed[u] + size[u] for u in clash)
+        placed[v] = off
+    total = max(placed[v] + size[v] for v in placed)
+    if total >= sum(size.values()):
+        return {}
+    return placed
+
+
+def _lds_regions(kernel: Kernel, plan: Dict[VarId, int]) -> Dict[VarId, Any]:
+    """Tiles that share bytes are one object for the hazard analysis."""
+    if not plan:
+        return {}
+    decl = {s.v: s for s in walk(kernel.body) if s.op == "declST"}
+    size = {v: (d.rows * (d.cols * _DTYPE_BYTES[d.dtype] + 16) + 15) // 16 * 16 for v, d in decl.items()}
+    root = {v: v for v in plan}
+
+    def find(v):
+        while root[v] != v:
+            v = root[v]
+        return v
+    vs = list(plan)
+    for i, a in enumerate(vs):
+        for b in vs[i + 1:]:
+            if plan[a] < plan[b] + size[b] and plan[b] < plan[a] + size[a]:
+                root[find(a)] = find(b)
+    return {v: ("lds", find(v).ident) for v in vs}
+
+
+def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None) -> set:
     """ids of the statements that need a workgroup barrier in front of them.
 
     Every wave of a workgroup runs the whole tile program, so the LDS tiles and vectors are shared
@@ -124,17 +217,21 @@ def shared_hazard_barriers(kernel: Kernel) -> set:
     after its own write.)  A conditional body cannot hold a barrier, so the barrier goes in front of
     the conditional."""
     shared = {s.v for s in walk(kernel.body) if s.op in ("declST", "declSV")}
+    regions = regions or {}
+
+    def obj(v):
+        return {regions.get(v, v)} if v in shared else set()
 
     def rw(s: Stmt):
         if s.op == "load":
-            return ({s.src} & shared, set())
+            return (obj(s.src), set())
         if s.op == "store":
-            return (set(), {s.dst} & shared)
+            return (set(), obj(s.dst))
         if s.op in ("loadGlobal", "loadVecGlobal", "loadVecGlobalCoord"):
-            return (set(), {s.dst} & shared)
+            return (set(), obj(s.dst))
         if s.op in ("storeGlobal", "storeVecGlobal", "storeVecGlobalCoord", "storeGlobalAdd", "storeVecGlobalAdd",
                     "storeVecGlobalAddCoord"):
-            return ({s.src} & shared, set())
+            return (obj(s.src), set())
         if s.op == "swapLayout" or (s.op == "transpose"):
             return ({("scratch", id(s))}, {("scratch", id(s))})      # the statement's own staging tile
         return (set(), set())
@@ -179,11 +276,16 @@ def shared_hazard_barriers(kernel: Kernel) -> set:
 
 class _Emitter:
     def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True,
-                 prefetch_global_loads: bool = True):
+                 prefetch_global_loads: bool = True, share_lds: bool = True):
         self.k = kernel
         # request the next iteration's global tiles of a loop before the work of the current one
         self.prefetch_global_loads = prefetch_global_loads
-        self.barrier_before = shared_hazard_barriers(kernel) if hazard_barriers else set()
+        # LDS tiles with disjoint live ranges share storage
+        # (only where that asks for no barrier the program does not already have)
+        self.lds = lds_plan(kernel) if share_lds else {}
+        if self.lds and shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds)) != shared_hazard_barriers(kernel):
+            self.lds = {}
+        self.barrier_before = shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds)) if hazard_barriers else set()
         # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
         # full 512-register file, and covers the 128-thread blocks the reference's runners launch
         self.max_waves = max_waves
@@ -210,7 +312,10 @@ class _Emitter:
         if op == "declRT":
             return f"{ind}rt<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)};\n"
         if op == "declST":
-            return f"{ind}__shared__ st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}> {I(s.v)};\n"
+            ty = f"st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}>"
+            if s.v in self.lds:
+                return f"{ind}{ty}& {I(s.v)} = *reinterpret_cast<{ty}*>(tyr_lds_pool + {self.lds[s.v]});\n"
+            return f"{ind}__shared__ {ty} {I(s.v)};\n"
         if op == "declRV":
             return f"{ind}rv<{_cpp_type(s.dtype)}, {s.len}, vlayout::{self.rv_layout[s.v]}> {I(s.v)};\n"
         if op == "declSV":
@@ -445,7 +550,14 @@ class _Emitter:
 
     def kernel_text(self) -> str:
         sig = ", ".join(t for t, _, _ in self.param_decls())
-        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" +
+        pool = ""
+        if self.lds:
+            decl = {t.v: t for t in walk(self.k.body) if t.op == "declST"}
+            total = max(off + (decl[v].rows * (decl[v].cols * _DTYPE_BYTES[decl[v].dtype] + 16) + 15) // 16 * 16
+                        for v, off in self.lds.items())
+            pool = (f"  // LDS tiles whose live ranges do not intersect share these bytes\n"
+                    f"  __shared__ __attribute__((aligned(16))) unsigned char tyr_lds_pool[{total}];\n")
+        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" + pool +
                 self.body(self.k.body, "  ") + "}\n")
 
     def launcher_signature(self) -> str:
@@ -563,9 +675,11 @@ def emit_header(kernels: List[Kernel], cites: Dict[str, str]) -> str:
     return out + "#ifdef __cplusplus\n}\n#endif\n\n#endif /* TYR_DSL_KERNELS_H */\n"
 
 
-def emit_kernel(kernel: Kernel, hazard_barriers: bool = True, prefetch_global_loads: bool = True) -> str:
+def emit_kernel(kernel: Kernel, hazard_barriers: bool = True, prefetch_global_loads: bool = True,
+                share_lds: bool = True) -> str:
     """Device code of one kernel (no includes)."""
-    return _Emitter(kernel, hazard_barriers=hazard_barriers, prefetch_global_loads=prefetch_global_loads).kernel_text()
+    return _Emitter(kernel, hazard_barriers=hazard_barriers, prefetch_global_loads=prefetch_global_loads,
+                    share_lds=share_lds).kernel_text()
 
 
 def emit_translation_unit(kernels: List[Kernel]) -> str:
