@@ -260,8 +260,12 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             // beside the exponentials of T=0, then the dQ products of T=0 beside the exponentials of T=1.
             f32x16 s[2], dp[2];
             bf16x8 dsf[4];
+            // the tile's 64 key-mask bytes as one word (bit r set: kv row j0 + r is hidden): one byte per
+            // lane and a ballot; a tile without hidden rows skips the masking
+            uint64_t tile_hidden = 0;
+            if (EXT && km != nullptr) tile_hidden = __builtin_amdgcn_ballot_w64(km[min(j0 + lane, N - 1)] == 0);
             const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
-                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && km != nullptr);
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && tile_hidden != 0);
             auto scores = [&](int T) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
@@ -281,18 +285,11 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
                     const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;
                     const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;
                     const int base = j0 + 4 * g;
-                    uint32_t hidden = 0;             // bit e: the key mask hides this lane's kv row
-                    if (EXT && km != nullptr) {
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                            hidden |= (km[min(kv, N - 1)] == 0 ? 1u : 0u) << e;
-                        }
-                    }
+                    const uint64_t hidden = tile_hidden >> (4 * g + 32 * T);      // shifted to this lane's rows
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        const bool off = kv > lim || (EXT && kv < low) || ((hidden >> e) & 1u);
+                        const bool off = kv > lim || (EXT && kv < low) || ((hidden >> (8 * (e >> 2) + (e & 3))) & 1u);
                         s[T][e] = off ? -INFINITY : s[T][e];
                     }
                 }
@@ -519,8 +516,10 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         }
     };
     // P and dS of half sh of a sub-tile (query rows qs0 + 16sh + 8h + 4g + x) as one k-step of column operands
+    // `apply` (wave-uniform) says whether any (query, key) pair of the rows at hand is hidden from this
+    // wave's keys; the mask instructions are skipped otherwise.
     auto probabilities = [&](auto masked, auto half, const f32x4 (&st)[4], int qs0, const f32x16& s, const f32x16& dp,
-                             bf16x8& pf, bf16x8& dsf) {
+                             bf16x8& pf, bf16x8& dsf, bool apply) {
         constexpr bool need_mask = decltype(masked)::value;
         constexpr int sh = decltype(half)::value;
         u32x4 ppk, dpk;
@@ -533,7 +532,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             float p[4], ds[4];
 #pragma unroll
             for (int x = 0; x < 4; ++x) p[x] = fast_exp2(fmaf(s[8 * sh + 4 * h + x], scale_log2, -l2[x]));
-            if (need_mask) {
+            if (need_mask && apply) {
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
                     const int qrow = qs0 + 8 * (2 * sh + h) + 4 * g + x;
@@ -568,6 +567,13 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         }
     };
 
+    // With EXT a step applies the mask only where some pair of the 64 query rows it touches (the second
+    // half of u, the first half of u+1) is hidden from this wave's keys: a key at or beyond the sequence's
+    // length or switched off by the key mask, the causal diagonal, the far edge of the window.
+    const bool wave_key_hidden = EXT && __builtin_amdgcn_ballot_w64(kvpos >= Nk || key_off) != 0;
+    auto rows_are_masked = [&](int qs0) {
+        return wave_key_hidden || (CAUSAL && qs0 < nw0 + 32) || (window > 0 && qs0 + 63 - nw0 >= window);
+    };
     bf16x8 rq[C::KSTEPS], rd[C::KSTEPS];              // row fragments of the next sub-tile, read one step ahead
     bf16x8 pf0, dsf0;                                 // P, dS of the first half of the current sub-tile
     f32x4 st1[4];                                     // pairs of its second half
@@ -595,7 +601,8 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
         read_transposed(stg, 2 * T + 1, dot1, qt1);
         scores(rq, rd, sn, dpn);
         bf16x8 pf1, dsf1;
-        probabilities(masked, Half1{}, st1, qs0, sc, dpc, pf1, dsf1);
+        const bool apply = decltype(masked)::value && rows_are_masked(qs0);       // rows qs0 .. qs0 + 63
+        probabilities(masked, Half1{}, st1, qs0, sc, dpc, pf1, dsf1, apply);
         read_pairs(Stg1{}, Sub1{}, Half1{}, st1);          // ahead of the row fragments: LDS answers in order
         read_rows(Stg2{}, sub, rq, rd);
 #pragma unroll
@@ -608,7 +615,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
             dv[dt] = mfma_32x32x16_bf16(dot1[dt], pf1, dv[dt]);
             dk[dt] = mfma_32x32x16_bf16(qt1[dt], dsf1, dk[dt]);
         }
-        probabilities(masked, Half0{}, st0, qs0 + 32, sn, dpn, pf0, dsf0);
+        probabilities(masked, Half0{}, st0, qs0 + 32, sn, dpn, pf0, dsf0, apply);
 #ifndef TYR_DKV_NO_SCHED
         // issue order: one MFMA, then its share of the LDS reads and of the vector work
 #pragma unroll
@@ -654,7 +661,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
                 if (kvpos > qs0 + 8 * (e >> 2) + 4 * g + (e & 3)) sc[e] = -INFINITY;
         }
         read_rows(Stg1{}, Sub1{}, rq, rd);
-        probabilities(masked, Half0{}, st0, qs0, sc, dpc, pf0, dsf0);
+        probabilities(masked, Half0{}, st0, qs0, sc, dpc, pf0, dsf0, true);
     };
 #undef TYR_STG
 

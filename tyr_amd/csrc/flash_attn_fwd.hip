@@ -261,30 +261,25 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
 
             // ---- mask (diagonal tiles, ragged tail) -- register e of sub-tile T is kv row
             //      j0 + 32T + 8(e/4) + 4g + e%4
+            // The tile's 64 key-mask bytes are the same for every lane: lane l reads the byte of kv row
+            // j0 + l and a ballot makes them one 64-bit word (bit r set: row j0 + r is hidden).  A tile
+            // without hidden rows skips the masking.  (Rows at or beyond N are hidden by `lim` already.)
+            uint64_t tile_hidden = 0;
+            if (EXT && km != nullptr) tile_hidden = __builtin_amdgcn_ballot_w64(km[min(j0 + lane, N - 1)] == 0);
             const bool need_mask = (CAUSAL && (j0 + BN - 1 > qw0)) || (j0 + BN > Nk) ||
-                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && km != nullptr);
+                                   (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && tile_hidden != 0);
             if (need_mask) {
                 const int lim = CAUSAL ? min(qpos, Nk - 1) : Nk - 1;   // largest visible kv row
                 const int low = (EXT && window > 0) ? qpos - window + 1 : INT_MIN;   // smallest visible kv row
                 const int base = j0 + 4 * g;
-                // bit 16T+e: the key mask hides this lane's kv row (gathered first, so that the
-                // masking below is one select per score)
-                uint32_t hidden = 0;
-                if (EXT && km != nullptr) {
-#pragma unroll
-                    for (int T = 0; T < 2; ++T)
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                            hidden |= (km[min(kv, N - 1)] == 0 ? 1u : 0u) << (16 * T + e);
-                        }
-                }
+                const uint64_t hidden = tile_hidden >> (4 * g);      // shifted to this lane's rows
 #pragma unroll
                 for (int T = 0; T < 2; ++T)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int kv = base + 32 * T + 8 * (e >> 2) + (e & 3);
-                        const bool off = kv > lim || (EXT && kv < low) || ((hidden >> (16 * T + e)) & 1u);
+                        const bool off = kv > lim || (EXT && kv < low) ||
+                                         ((hidden >> (32 * T + 8 * (e >> 2) + (e & 3))) & 1u);
                         cur[T][e] = off ? -INFINITY : cur[T][e];
                     }
             }
