@@ -247,8 +247,8 @@ def wl_gemm_bf16(torch, tyr, steps, warmup, cpu):
 def wl_gemm_fp8(torch, tyr, steps, warmup, cpu):
     M = N = K = 8192
     torch.manual_seed(3)
-    aq, sa = tyr.quantize_e4m3(torch.randn(M, K, device="cuda"))
-    bq, sb = tyr.quantize_e4m3(torch.randn(K, N, device="cuda"))
+    aq, sa = tyr.quantize_e4m3(_normal(torch, M, K))
+    bq, sb = tyr.quantize_e4m3(_normal(torch, K, N))
     fn = lambda: tyr.gemm_fp8(aq, bq, sa, sb)
     wall, ms = time_steps(torch, fn, steps, warmup)
     tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
@@ -444,7 +444,7 @@ def main() -> int:
     ap.add_argument("--settle-ms", type=float, default=PREWARM_MS,
                     help="untimed work before the warm-up steps of every workload, in milliseconds")
     ap.add_argument("--data", default="randn", choices=["randn", "constant"],
-                    help="operand values of the attention and bf16 GEMM workloads; 'constant' is a power diagnostic")
+                    help="operand values of the attention and GEMM workloads; 'constant' is a power diagnostic")
     args = ap.parse_args()
     globals()["PREWARM_MS"] = args.settle_ms
     globals()["DATA"] = args.data
