@@ -226,15 +226,19 @@ __global__ __launch_bounds__(D) void gqa_decode_combine_kernel(
     const float* pl = part_l + (size_t)bh * S;
     const float* po = part_o + (size_t)bh * S * D + d;
     float m = -INFINITY;
+#pragma unroll 8
     for (int s = 0; s < S; ++s) m = fmaxf(m, pm[s]);
+    // The loads of a partial do not depend on its weight, so eight splits are in flight at a time
+    // (an empty split's O is never written: it is read and discarded, not multiplied).
     float o = 0.0f, l = 0.0f;
+#pragma unroll 8
     for (int s = 0; s < S; ++s) {
         const float ms = pm[s];
-        if (ms > -INFINITY) {
-            const float wgt = fast_exp2(ms - m);
-            o += po[(size_t)s * D] * wgt;
-            l += pl[s] * wgt;
-        }
+        const float os = po[(size_t)s * D], ls = pl[s];
+        const bool live = ms > -INFINITY;
+        const float wgt = live ? fast_exp2(ms - m) : 0.0f;
+        o += live ? os * wgt : 0.0f;
+        l += live ? ls * wgt : 0.0f;
     }
     const float res = o / l;
     // pairs of threads pack two bf16 into one dword
