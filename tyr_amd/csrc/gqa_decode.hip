@@ -160,10 +160,12 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
             oacc[j] = mfma_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt[j]), pfrag, oacc[j]);
     };
 
-#pragma unroll
-    for (int i = 0; i < KI; ++i) pin_registers(qf[i]);
+    // the first K / V rows are requested before Q is waited for (loads return in order: waiting for
+    // the older Q does not wait for them)
     Buf<D> b0, b1;
     if (nsteps > 0) load(b0, r0);
+#pragma unroll
+    for (int i = 0; i < KI; ++i) pin_registers(qf[i]);
     for (int st = 0; st < nsteps; st += 2) {
         if (st + 1 < nsteps) load(b1, r0 + (st + 1) * SST);
         compute(b0, r0 + st * SST);
