@@ -747,7 +747,7 @@ int launch_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     const int ntq = (N + 127) / 128;
     const int npad = ntq * 128;
     const bool ext = window > 0 || kv_lens != nullptr || key_mask != nullptr;
-    const int pair = (causal && !ext && ntq > 1) ? 1 : 0;
+    const int pair = (causal && window <= 0 && ntq > 1) ? 1 : 0;   // lengths and key masks keep tile 0 starting at key 0
     dim3 grid_q((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), grid_k((unsigned)(BHkv * ntq)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
