@@ -381,6 +381,36 @@ def test_flash_attn_arbitrary_key_mask_matches_oracle(gpu, B, Hq, Hkv, N, D, cau
     assert max_abs(o1.cpu().float(), o0.cpu().float()) <= 1e-2 and max_abs(l1.cpu(), l0.cpu()) <= 1e-3
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_attn_key_mask_with_whole_tiles_hidden(gpu, causal):
+    # key tiles of 64 rows that are wholly hidden, wholly visible (those skip the masking) or mixed, over
+    # several query tiles (the paired causal schedule); forward and backward against the checker
+    B, Hq, Hkv, N, D = 2, 4, 2, 448, 128
+    q, g_ = lt.make_inputs(931, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(932, (B, Hkv, N, D), (B, Hkv, N, D))
+    km = torch.ones(B, N, dtype=torch.bool)
+    km[0, 64:192] = False                  # two whole tiles
+    km[0, 300:310] = False                 # a hole inside a tile
+    km[1, :128] = False                    # left padding of two tiles: causal rows there see nothing
+    km[1, 400:] = False                    # and a hidden tail
+    sc = 1.0 / math.sqrt(D)
+    o, lse = gpu.flash_attn_fwd(q.cuda(), k.cuda(), v.cuda(), causal=causal, scale=sc, key_mask=km.cuda())
+    want_o, want_lse = oracle.attn_fwd_f64_ex(bits(q), bits(k), bits(v), causal, sc, key_mask=km.numpy())
+    dead = np.isneginf(want_lse)
+    assert max_abs(o.cpu().float(), want_o) <= 2e-2
+    assert np.array_equal(np.isneginf(lse.cpu().numpy()), dead)
+    assert float(np.abs(lse.cpu().numpy()[~dead] - want_lse[~dead]).max()) <= 2e-2
+    dq, dk, dv = gpu.flash_attn_bwd(q.cuda(), k.cuda(), v.cuda(), o, lse, g_.cuda(), causal=causal, scale=sc,
+                                    key_mask=km.cuda())
+    wq, wk, wv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g_), causal, sc, key_mask=km.numpy())
+    for got, want in ((dq, wq), (dk, wk), (dv, wv)):
+        got = got.cpu().float().numpy()
+        assert np.all(np.abs(got - want) <= 3e-2 + 3e-2 * np.abs(want))
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-2
+    hidden = ~km.numpy()
+    assert float(np.abs(dk.cpu().float().numpy()[hidden[:, None, :].repeat(Hkv, 1)]).max()) == 0.0   # hidden keys get no gradient
+
+
 def test_flash_attn_key_mask_argument_checks(gpu):
     q, k, v = (t.cuda() for t in lt.make_inputs(5, (1, 2, 64, 64), (1, 2, 64, 64), (1, 2, 64, 64)))
     with pytest.raises(gpu.TyrGpuError, match="shape"):
