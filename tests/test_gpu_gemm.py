@@ -25,7 +25,9 @@ def gpu():
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 512, 4096), (8, 8, 8),
                                    (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256), (768, 512, 320),
-                                   (300, 264, 128), (1, 16, 64), (513, 520, 192), (700, 1000, 256)])
+                                   (300, 264, 128), (1, 16, 64), (513, 520, 192), (700, 1000, 256),
+                                   # K with a last slice shorter than 64: its chunks past K are the next row's data
+                                   (64, 64, 40), (129, 80, 1000), (512, 512, 4000)])
 def test_gemm_bf16_matches_oracle(gpu, M, N, K, trans_b):
     a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
     bb = b.t().contiguous() if trans_b else b
@@ -128,7 +130,9 @@ def test_gemm_bf16_full_size_config(gpu):
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 256, 384), (16, 16, 16), (300, 272, 80),
                                    (1, 16, 16), (257, 48, 1040), (768, 512, 640),
-                                   (300, 272, 128), (1, 16, 128), (513, 528, 384), (700, 1008, 256)])
+                                   (300, 272, 128), (1, 16, 128), (513, 528, 384), (700, 1008, 256),
+                                   # K with a last slice shorter than 128
+                                   (64, 64, 48), (129, 80, 1008), (512, 512, 4000)])
 def test_gemm_fp8_matches_oracle(gpu, M, N, K, trans_b):
     torch.manual_seed(200 + M + N + K)
     a, b = torch.randn(M, K), torch.randn(K, N)

@@ -123,7 +123,10 @@ __device__ __forceinline__ u32x2 ds_read_tr8(const void* lds_ptr) {
 }
 
 // Buffer resource (V#) for raw byte-addressed access to [base, base + bytes): loads beyond the
-// range return zero.
+// range return zero.  On gfx950 the range check covers the whole offset, per-lane, scalar and immediate
+// parts together (probed with a 4 KiB descriptor inside a larger allocation: a scalar offset of 4000
+// gives data to the lanes below byte 4096 and zeros to the rest), so a slice index carried in the
+// scalar offset is zero-filled past the end like a row index carried in the per-lane offset.
 __device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, uint32_t bytes) {
     const uint64_t a = reinterpret_cast<uint64_t>(base);
     return u32x4{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};

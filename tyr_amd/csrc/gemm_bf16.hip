@@ -181,7 +181,7 @@ __global__ __launch_bounds__(gemm::THREADS) void gemm_bf16_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path for K % 64 == 0 (any M; N % 8 == 0).
+// Fast path for K % 8 == 0 (any M; N % 8 == 0; a last slice shorter than 64 is zero-filled).
 //
 // Same 256x256x64 decomposition, but the slices travel from global memory straight into LDS
 // (no register staging, no LDS stores from the ALU), rows are unpadded with XOR-swizzled 16-byte
@@ -197,7 +197,7 @@ constexpr int LDS_BYTES = 2 * STAGE;                 // 128 KiB
 constexpr int GROUP_M = 4;
 }  // namespace gemm2
 
-template <bool TRANS_B>
+template <bool TRANS_B, bool K_TAIL>
 __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, int tiles_m, int tiles_n) {
@@ -223,9 +223,11 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     // A (and B when TRANS_B): 8 rows of 128 B per instruction; chunk c of row m is stored at
     // position c ^ ((m >> 1) & 7), so 16 consecutive rows put one logical chunk on all 64 banks.  B when !TRANS_B: 2 rows of 512 B per instruction; chunk c of row k is
     // stored at position c ^ ((k & 3) << 2).
-    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K * 2, (size_t)0xffffffffu));
+    // (a descriptor spans the tile's rows only and stays below 2 GiB, so that the offset 2^31 given to
+    //  the chunks past K of a ragged last slice is out of range whatever is added to it)
+    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)((size_t)min(M - m0, BM) * K * 2));
     const u32x4 b_rsrc = TRANS_B
-        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K * 2, (size_t)0xffffffffu))
+        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)((size_t)min(N - n0, BN) * K * 2))
         // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
         //  off the per-lane offsets below, and those must not go negative)
         : make_raw_rsrc(B + n0 - 1536, (uint32_t)min(((size_t)K * N - n0) * 2 + 3072, (size_t)0xffffffffu));
@@ -248,12 +250,27 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
     // half h (0..1) of the requests for slice kt into stage st: 4 A + 4 B instructions, each group of
     // four behind one M0 write (the immediate offset steps the LDS destination by a kilobyte)
+    const int KT = (K + BK - 1) / BK;
     auto issue_half = [&](int st, int kt, int h) {
         const int a_soff = kt * BK * 2;
         const int b_soff = TRANS_B ? kt * BK * 2 : kt * BK * N * 2;
         const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
-        const int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
-        const int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
+        int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        if (K_TAIL && kt == KT - 1) {
+            // ragged last slice (K % 8 == 0): the 16-byte chunks of a row at k >= K belong to the next
+            // row and must read as zeros; rows k >= K of a [K,N] B are past its descriptor already
+            const int chunks = (K - kt * BK) >> 3;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = (w * 8 + 4 * h + i) * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((row >> 1) & 7);
+                if (c >= chunks) {
+                    av[i] = (int)0x80000000u;
+                    if (TRANS_B) bv[i] = (int)0x80000000u;
+                }
+            }
+        }
         load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
         load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
@@ -306,7 +323,6 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         }
     };
 
-    const int KT = K / BK;
 #pragma unroll
     for (int h = 0; h < 2; ++h) issue_half(0, 0, h);
     wait_vmcnt0();
@@ -357,22 +373,24 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
     auto Bp = static_cast<const uint16_t*>(b);
     auto Cp = static_cast<uint16_t*>(c);
     // 32-bit buffer offsets: one 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
-    // The fast kernel needs whole K slices; ragged M and N are handled by the zero fill of the
-    // buffer loads (rows past the end) and by the guarded epilogue (columns past N only ever
-    // contribute to outputs that are not stored).
-    const bool fast_ok = (K % BK == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
+    // The fast kernel needs rows of whole 16-byte chunks; ragged M, N and K are handled by the zero
+    // fill of the buffer loads (rows past the end, chunks past K) and by the guarded epilogue (columns
+    // past N only ever contribute to outputs that are not stored).
+    const bool fast_ok = (K % 8 == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N * 2 < ((size_t)1 << 32));
     if (fast_ok) {
-#define TYR_GEMM_FAST(TB)                                                                         \
+#define TYR_GEMM_FAST(TB, KT)                                                                     \
         do {                                                                                      \
             static const hipError_t attr = hipFuncSetAttribute(                                   \
-                reinterpret_cast<const void*>(&gemm_bf16_fast_kernel<TB>),                        \
+                reinterpret_cast<const void*>(&gemm_bf16_fast_kernel<TB, KT>),                    \
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm2::LDS_BYTES);                    \
             if (attr != hipSuccess) return -1;                                                    \
-            hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB>), grid, block, gemm2::LDS_BYTES, stream, \
+            hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB, KT>), grid, block, gemm2::LDS_BYTES, stream, \
                                A, Bp, Cp, M, N, K, tiles_m, tiles_n);                             \
         } while (0)
-        if (trans_b) TYR_GEMM_FAST(true); else TYR_GEMM_FAST(false);
+        const bool k_tail = K % gemm2::BK != 0;
+        if (trans_b) { if (k_tail) TYR_GEMM_FAST(true, true); else TYR_GEMM_FAST(true, false); }
+        else         { if (k_tail) TYR_GEMM_FAST(false, true); else TYR_GEMM_FAST(false, false); }
 #undef TYR_GEMM_FAST
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }

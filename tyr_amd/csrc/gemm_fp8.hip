@@ -198,7 +198,7 @@ __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path for K % 128 == 0 (any M; N % 16 == 0): slices go from global memory straight
+// Fast path for K % 16 == 0 (any M; N % 16 == 0; a last slice shorter than 128 is zero-filled): slices go from global memory straight
 // into LDS, unpadded rows with XOR-swizzled 16-byte chunks; a [K,N] B stays row-major in LDS and
 // its fragments (32 consecutive k for one n) are gathered with the byte-transposing LDS read.
 namespace gemm8f {
@@ -210,7 +210,7 @@ constexpr int LDS_BYTES = 2 * STAGE;
 constexpr int GROUP_M = 4;
 }  // namespace gemm8f
 
-template <bool TRANS_B>
+template <bool TRANS_B, bool K_TAIL>
 __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, int tiles_m, int tiles_n, float scale) {
@@ -235,9 +235,11 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     // ---- global -> LDS requests (8 instructions of 1 KiB per wave and tile).
     // A (and B when TRANS_B): 8 rows of 128 B per instruction, chunk c of row m at c ^ ((m>>1)&7).
     // B when !TRANS_B: 4 rows of 256 B per instruction, chunk c of row k at c ^ ((k&7)<<1).
-    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((size_t)(M - m0) * K, (size_t)0xffffffffu));
+    // (a descriptor spans the tile's rows only and stays below 2 GiB, so that the offset 2^31 given to
+    //  the chunks past K of a ragged last slice is out of range whatever is added to it)
+    const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)((size_t)min(M - m0, BM) * K));
     const u32x4 b_rsrc = TRANS_B
-        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((size_t)(N - n0) * K, (size_t)0xffffffffu))
+        ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)((size_t)min(N - n0, BN) * K))
         // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
         //  off the per-lane offsets below, and those must not go negative)
         : make_raw_rsrc(B + n0 - 3072, (uint32_t)min((size_t)K * N - n0 + 3072, (size_t)0xffffffffu));
@@ -258,13 +260,28 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
+    const int KT = (K + BK - 1) / BK;
     auto issue_half = [&](int st, int kt, int h) {
         const int a_soff = kt * BK;
         const int b_soff = TRANS_B ? kt * BK : kt * BK * N;
         // four requests behind one M0 write: the immediate offset steps the LDS destination by a kilobyte
         const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
-        const int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
-        const int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
+        int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        if (K_TAIL && kt == KT - 1) {
+            // ragged last slice (K % 16 == 0): the 16-byte chunks of a row at k >= K belong to the next
+            // row and must read as zeros; rows k >= K of a [K,N] B are past its descriptor already
+            const int chunks = (K - kt * BK) >> 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = (w * 8 + 4 * h + i) * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((row >> 1) & 7);
+                if (c >= chunks) {
+                    av[i] = (int)0x80000000u;
+                    if (TRANS_B) bv[i] = (int)0x80000000u;
+                }
+            }
+        }
         load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
         load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
@@ -332,7 +349,6 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
         }
     };
 
-    const int KT = K / BK;
     issue_half(0, 0, 0);
     issue_half(0, 0, 1);
     wait_vmcnt0();
@@ -382,19 +398,21 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
     // 32-bit buffer offsets: a 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
     // The fast kernel needs whole K slices; ragged M and N are handled by the zero fill of the
     // buffer loads and by the guarded epilogue.
-    const bool fast_ok = (K % BK == 0) && (size_t)256 * K < ((size_t)1 << 31) &&
+    const bool fast_ok = (K % 16 == 0) && (size_t)256 * K < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N < ((size_t)1 << 32));
     if (fast_ok) {
-#define TYR_GEMM8_FAST(TB)                                                                        \
+#define TYR_GEMM8_FAST(TB, KT)                                                                      \
         do {                                                                                      \
             static const hipError_t attr = hipFuncSetAttribute(                                   \
-                reinterpret_cast<const void*>(&gemm_fp8_fast_kernel<TB>),                         \
+                reinterpret_cast<const void*>(&gemm_fp8_fast_kernel<TB, KT>),                     \
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm8f::LDS_BYTES);                   \
             if (attr != hipSuccess) return -1;                                                    \
-            hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB>), grid, block, gemm8f::LDS_BYTES, stream, \
+            hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB, KT>), grid, block, gemm8f::LDS_BYTES, stream, \
                                A, Bp, Cp, M, N, K, tiles_m, tiles_n, scale);                      \
         } while (0)
-        if (trans_b) TYR_GEMM8_FAST(true); else TYR_GEMM8_FAST(false);
+        const bool k_tail = K % gemm8f::BK != 0;
+        if (trans_b) { if (k_tail) TYR_GEMM8_FAST(true, true); else TYR_GEMM8_FAST(true, false); }
+        else         { if (k_tail) TYR_GEMM8_FAST(false, true); else TYR_GEMM8_FAST(false, false); }
 #undef TYR_GEMM8_FAST
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }
