@@ -278,6 +278,9 @@ int tyr_hip_copy(const void* src, void* dst, size_t bytes, void* stream);
  *
  *   a : bf16 [M, K]   b : bf16 [K, N] or [N, K]   c : bf16 [M, N]
  * Supported: M, N, K >= 1 with K % 8 == 0 and N % 8 == 0 (16-byte rows).
+ * With TYR_HIP_GEMM_GENERAL set in the environment, this and the fp8 GEMM run their general
+ * (register-staged) kernels on every shape; unset, only shapes whose 256-row panels or whose [K, N]
+ * B exceed 32-bit byte offsets do.  The switch exists for tests and for comparing the two paths.
  */
 int tyr_hip_gemm_bf16(const void* a, const void* b, void* c,
                       uint64_t M, uint64_t N, uint64_t K, int trans_b, void* stream);

@@ -73,6 +73,40 @@ def test_gemm_random_shapes(gpu, seed):
 
 
 @pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (300, 264, 72), (1, 16, 8), (257, 8, 520)])
+def test_gemm_general_kernels_match_oracle(gpu, monkeypatch, M, N, K, trans_b):
+    # The general (register-staged) kernels serve shapes beyond the fast kernels' 32-bit offsets;
+    # the environment switch sends ordinary shapes through them.
+    monkeypatch.setenv("TYR_HIP_GEMM_GENERAL", "1")
+    a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
+    bb = b.t().contiguous() if trans_b else b
+    c = gpu.gemm_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
+    assert rel_fro(c, a.float() @ b.float()) <= TOL_FRO
+    want = from_bits(oracle.gemm_bf16(bits(a), bits(bb), trans_b=trans_b)).float()
+    assert (c.float() - want).abs().max() <= 2.0 ** -7 * want.abs().max()
+    K8 = (K + 15) // 16 * 16
+    torch.manual_seed(M + N + K8)
+    a8, b8 = torch.randn(M, K8), torch.randn(K8, N - N % 16 + 16)
+    aq, sa = lt.quantize_e4m3(a8)
+    bq, sb = lt.quantize_e4m3(b8)
+    bqb = bq.t().contiguous() if trans_b else bq
+    c8 = gpu.gemm_fp8(aq.cuda(), bqb.cuda(), sa, sb, trans_b=trans_b).cpu()
+    assert rel_fro(c8, lt.fp8_mm(aq, bq, sa, sb)) <= TOL_FRO
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gemm_rows_longer_than_the_fast_kernels_offsets(gpu, trans_b):
+    # 256 rows of K elements no longer fit a 31-bit byte offset: the launcher takes the general kernel.
+    M, N, K = 8, 16, 1 << 22
+    g = torch.Generator().manual_seed(5)
+    a = (torch.randn(M, K, generator=g) * K ** -0.25).to(torch.bfloat16)
+    b = (torch.randn(K, N, generator=g) * K ** -0.25).to(torch.bfloat16)
+    bb = b.t().contiguous() if trans_b else b
+    c = gpu.gemm_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
+    assert rel_fro(c, a.double() @ b.double()) <= TOL_FRO
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(300, 264, 128), (257, 8, 64), (1, 272, 256), (511, 504, 72)])
 def test_gemm_ragged_tiles_write_only_c(gpu, M, N, K, trans_b):
     # C sits inside a larger buffer of a canary value: tiles that overhang M or N must not

@@ -16,6 +16,7 @@
 //     multiplied, then written to the other stage: one barrier per slice.
 //   * The MFMA is issued with the B fragment as its row operand, so every lane ends up with
 //     4 consecutive n for one m and stores 8-byte pieces of a C row.
+#include <cstdlib>
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -376,7 +377,10 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
     // The fast kernel needs rows of whole 16-byte chunks; ragged M, N and K are handled by the zero
     // fill of the buffer loads (rows past the end, chunks past K) and by the guarded epilogue (columns
     // past N only ever contribute to outputs that are not stored).
-    const bool fast_ok = (K % 8 == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
+    // TYR_HIP_GEMM_GENERAL (any value) sends every shape to the general kernels, which otherwise only
+    // shapes beyond the 32-bit offsets reach: a switch for tests and for comparing the two paths.
+    const bool general_only = std::getenv("TYR_HIP_GEMM_GENERAL") != nullptr;
+    const bool fast_ok = !general_only && (K % 8 == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N * 2 < ((size_t)1 << 32));
     if (fast_ok) {
 #define TYR_GEMM_FAST(TB, KT)                                                                     \
