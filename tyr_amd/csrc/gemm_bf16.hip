@@ -307,20 +307,16 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    auto read_frags = [&](const unsigned char* St, int s, bf16x8 (&af)[4], bf16x8 (&bf)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(St + a_roff[s] + i * 32 * 128);
+    // fragment pair i of k-step s: the A fragment of m tile i and the B fragment of n tile i
+    auto read_pair = [&](const unsigned char* St, int s, int i, bf16x8& fa, bf16x8& fb) {
+        fa = *reinterpret_cast<const bf16x8*>(St + a_roff[s] + i * 32 * 128);
         if (TRANS_B) {
-#pragma unroll
-            for (int jt = 0; jt < 4; ++jt) bf[jt] = *reinterpret_cast<const bf16x8*>(St + b_roff[s] + jt * 32 * 128);
+            fb = *reinterpret_cast<const bf16x8*>(St + b_roff[s] + i * 32 * 128);
         } else {
-#pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                const unsigned char* p = St + b_roff[jt] + s * 16 * 512;
-                const bf16x4 lo = ds_read_tr16(p);
-                const bf16x4 hi = ds_read_tr16(p + 4 * 512);
-                bf[jt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
+            const unsigned char* p = St + b_roff[i] + s * 16 * 512;
+            const bf16x4 lo = ds_read_tr16(p);
+            const bf16x4 hi = ds_read_tr16(p + 4 * 512);
+            fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
     };
 
@@ -329,34 +325,50 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     wait_vmcnt0();
     __syncthreads();
 
-    // Steady state per slice: the next slice is requested during k-steps 0 and 1; fragments for
-    // k-step s+1 are read before the MFMAs of k-step s; before the MFMAs of the last k-step the
-    // workgroup synchronises and already reads the first fragments of the next slice, so the
-    // barrier and the LDS latency hide under 16 MFMAs.  (Past the last slice the requests and
-    // reads touch the idle stage / stale data and are never used.)
+    // Steady state per slice: the next slice is requested during k-steps 0 and 1; the fragments of
+    // k-step s+1 are read during the MFMAs of k-step s; after the first MFMA row of the last k-step
+    // the workgroup synchronises and reads the first fragments of the next slice.  A wave is alone
+    // on its SIMD, so whatever it issues between two MFMAs is time the matrix pipe may idle: the
+    // requests and the fragment reads are dealt out between the MFMA rows (4 MFMAs, 128 cycles each)
+    // instead of standing in one block before them, and the scheduling barriers keep that order.
+    // (Past the last slice the requests and reads touch the idle stage / stale data and are never used.)
     bf16x8 af[2][4], bf[2][4];
-    read_frags(lds, 0, af[0], bf[0]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) read_pair(lds, 0, i, af[0][i], bf[0][i]);
+#define TYR_FENCE __builtin_amdgcn_sched_barrier(0)
     for (int kt = 0; kt < KT; ++kt) {
         const int st = kt & 1;
         const unsigned char* St = lds + st * STAGE;
+        const unsigned char* Sn = lds + (st ^ 1) * STAGE;
+        auto row = [&](int b, int i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[b][j], af[b][i], acc[i][j]);
+        };
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            if (s < 2) issue_half(st ^ 1, kt + 1, s);
+            const int cb = s & 1, nb = cb ^ 1;
             if (s < 3) {
-                read_frags(St, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                if (s < 2) issue_half(st ^ 1, kt + 1, s);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    read_pair(St, s + 1, i, af[nb][i], bf[nb][i]);
+                    TYR_FENCE; row(cb, i); TYR_FENCE;
+                }
             } else {
+                row(cb, 0); TYR_FENCE;
                 wait_vmcnt0();
                 __syncthreads();
-                read_frags(lds + (st ^ 1) * STAGE, 0, af[0], bf[0]);
+                read_pair(Sn, 0, 0, af[nb][0], bf[nb][0]);
+                read_pair(Sn, 0, 1, af[nb][1], bf[nb][1]);
+                TYR_FENCE; row(cb, 1); TYR_FENCE;
+                read_pair(Sn, 0, 2, af[nb][2], bf[nb][2]);
+                read_pair(Sn, 0, 3, af[nb][3], bf[nb][3]);
+                TYR_FENCE; row(cb, 2); TYR_FENCE;
+                row(cb, 3); TYR_FENCE;
             }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[s & 1][j], af[s & 1][i], acc[i][j]);
-            __builtin_amdgcn_sched_barrier(0);
         }
     }
+#undef TYR_FENCE
 
     // ---- epilogue (all requests have landed and every wave is past its last fragment read)
     store_quadrant_bf16(acc, 1.0f, lds + w * kEpilogueScratchBytes,

@@ -323,64 +323,65 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    auto read_frags = [&](const unsigned char* St, int s, i32x8 (&af)[4], i32x8 (&bf)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + a_roff[s][0] + i * 32 * 128);
-            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + a_roff[s][1] + i * 32 * 128);
-            af[i] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-        }
-        if (TRANS_B) {
-#pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s] + jt * 32 * 128);
-                const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s + 1] + jt * 32 * 128);
-                bf[jt] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-            }
-        } else {
-#pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                const unsigned char* p = St + b_roff[jt] + s * 64 * 256;
-                const u32x2 y0 = ds_read_tr8(p);
-                const u32x2 y1 = ds_read_tr8(p + 8 * 256);
-                const u32x2 y2 = ds_read_tr8(p + 16 * 256);
-                const u32x2 y3 = ds_read_tr8(p + 24 * 256);
-                bf[jt] = i32x8{(int)y0.x, (int)y0.y, (int)y1.x, (int)y1.y, (int)y2.x, (int)y2.y, (int)y3.x, (int)y3.y};
-            }
-        }
-    };
-
     issue_half(0, 0, 0);
     issue_half(0, 0, 1);
     wait_vmcnt0();
     __syncthreads();
 
-    // Per slice: k-step 0 requests the next slice and reads the fragments of k-step 1; before the
-    // MFMAs of k-step 1 the workgroup synchronises and reads the first fragments of the next slice.
+    // Per slice: k-step 0 requests the next slice and reads the fragments of k-step 1; after the
+    // first MFMA row of k-step 1 the workgroup synchronises and reads the first fragments of the
+    // next slice.  A wave is alone on its SIMD, so whatever it issues between two MFMAs is time the
+    // matrix pipe may idle: the requests and the fragment reads are therefore dealt out between the
+    // MFMA rows (4 MFMAs, 256 cycles each) instead of standing in one block before them, and the
+    // scheduling barriers keep that order.
     i32x8 af[2][4], bf[2][4];
-    read_frags(lds, 0, af[0], bf[0]);
+    // fragment pair i of k-step s: the A fragment of m tile i and the B fragment of n tile i
+    auto read_pair = [&](const unsigned char* St, int s, int i, i32x8& a, i32x8& b) {
+        {
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + a_roff[s][0] + i * 32 * 128);
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + a_roff[s][1] + i * 32 * 128);
+            a = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        }
+        if (TRANS_B) {
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s] + i * 32 * 128);
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s + 1] + i * 32 * 128);
+            b = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        } else {
+            const unsigned char* p = St + b_roff[i] + s * 64 * 256;
+            const u32x2 y0 = ds_read_tr8(p);
+            const u32x2 y1 = ds_read_tr8(p + 8 * 256);
+            const u32x2 y2 = ds_read_tr8(p + 16 * 256);
+            const u32x2 y3 = ds_read_tr8(p + 24 * 256);
+            b = i32x8{(int)y0.x, (int)y0.y, (int)y1.x, (int)y1.y, (int)y2.x, (int)y2.y, (int)y3.x, (int)y3.y};
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) read_pair(lds, 0, i, af[0][i], bf[0][i]);
+#define TYR_FENCE __builtin_amdgcn_sched_barrier(0)
     for (int kt = 0; kt < KT; ++kt) {
         const int st = kt & 1;
         const unsigned char* St = lds + st * STAGE;
+        const unsigned char* Sn = lds + (st ^ 1) * STAGE;
+        auto row = [&](int s, int i) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            if (s == 0) {
-                issue_half(st ^ 1, kt + 1, 0);
-                issue_half(st ^ 1, kt + 1, 1);
-                read_frags(St, 1, af[1], bf[1]);
-            } else {
-                wait_vmcnt0();
-                __syncthreads();
-                read_frags(lds + (st ^ 1) * STAGE, 0, af[0], bf[0]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
+        };
+        issue_half(st ^ 1, kt + 1, 0);
+        read_pair(St, 1, 0, af[1][0], bf[1][0]); TYR_FENCE; row(0, 0); TYR_FENCE;
+        issue_half(st ^ 1, kt + 1, 1);
+        read_pair(St, 1, 1, af[1][1], bf[1][1]); TYR_FENCE; row(0, 1); TYR_FENCE;
+        read_pair(St, 1, 2, af[1][2], bf[1][2]); TYR_FENCE; row(0, 2); TYR_FENCE;
+        read_pair(St, 1, 3, af[1][3], bf[1][3]); TYR_FENCE; row(0, 3); TYR_FENCE;
+        row(1, 0); TYR_FENCE;
+        wait_vmcnt0();
+        __syncthreads();
+        read_pair(Sn, 0, 0, af[0][0], bf[0][0]);
+        read_pair(Sn, 0, 1, af[0][1], bf[0][1]); TYR_FENCE; row(1, 1); TYR_FENCE;
+        read_pair(Sn, 0, 2, af[0][2], bf[0][2]);
+        read_pair(Sn, 0, 3, af[0][3], bf[0][3]); TYR_FENCE; row(1, 2); TYR_FENCE;
+        row(1, 3); TYR_FENCE;
     }
+#undef TYR_FENCE
 
     store_quadrant_bf16(acc, scale, lds + w * kEpilogueScratchBytes,
                         C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
