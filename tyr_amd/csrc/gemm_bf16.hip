@@ -252,7 +252,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     // half h (0..1) of the requests for slice kt into stage st: 4 A + 4 B instructions, each group of
     // four behind one M0 write (the immediate offset steps the LDS destination by a kilobyte)
     const int KT = (K + BK - 1) / BK;
-    auto issue_half = [&](int st, int kt, int h) {
+    auto issue_half = [&](int st, int kt, int h, int part = 2) {
         const int a_soff = kt * BK * 2;
         const int b_soff = TRANS_B ? kt * BK * 2 : kt * BK * N * 2;
         const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
@@ -272,8 +272,8 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
                 }
             }
         }
-        load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
-        load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
+        if (part != 1) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        if (part != 0) load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses
@@ -348,9 +348,9 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         for (int s = 0; s < 4; ++s) {
             const int cb = s & 1, nb = cb ^ 1;
             if (s < 3) {
-                if (s < 2) issue_half(st ^ 1, kt + 1, s);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    if (s < 2 && i < 2) issue_half(st ^ 1, kt + 1, s, i);
                     read_pair(St, s + 1, i, af[nb][i], bf[nb][i]);
                     TYR_FENCE; row(cb, i); TYR_FENCE;
                 }

@@ -262,7 +262,7 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
     const int KT = (K + BK - 1) / BK;
-    auto issue_half = [&](int st, int kt, int h) {
+    auto issue_half = [&](int st, int kt, int h, int part = 2) {
         const int a_soff = kt * BK;
         const int b_soff = TRANS_B ? kt * BK : kt * BK * N;
         // four requests behind one M0 write: the immediate offset steps the LDS destination by a kilobyte
@@ -283,8 +283,8 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
                 }
             }
         }
-        load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
-        load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
+        if (part != 1) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        if (part != 0) load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses.  k-step s covers bytes [64s, 64s+64) of a row; lane group g takes
@@ -366,11 +366,13 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
         };
-        issue_half(st ^ 1, kt + 1, 0);
+        issue_half(st ^ 1, kt + 1, 0, 0);
         read_pair(St, 1, 0, af[1][0], bf[1][0]); TYR_FENCE; row(0, 0); TYR_FENCE;
-        issue_half(st ^ 1, kt + 1, 1);
+        issue_half(st ^ 1, kt + 1, 0, 1);
         read_pair(St, 1, 1, af[1][1], bf[1][1]); TYR_FENCE; row(0, 1); TYR_FENCE;
+        issue_half(st ^ 1, kt + 1, 1, 0);
         read_pair(St, 1, 2, af[1][2], bf[1][2]); TYR_FENCE; row(0, 2); TYR_FENCE;
+        issue_half(st ^ 1, kt + 1, 1, 1);
         read_pair(St, 1, 3, af[1][3], bf[1][3]); TYR_FENCE; row(0, 3); TYR_FENCE;
         row(1, 0); TYR_FENCE;
         wait_vmcnt0();
