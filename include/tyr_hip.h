@@ -163,6 +163,29 @@ int tyr_hip_gqa_decode(const void* q, const void* k, const void* v, void* o, flo
                        uint64_t kv_stride, float scale, uint64_t num_splits,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* tyr_hip_gqa_decode without a workspace argument and without any allocation.
+ *
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory around
+ * the call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The partial results of the split pass go to a fixed device array of
+ * TYR_HIP_GQA_DECODE_STATIC_SCRATCH_BYTES bytes that the library holds on every GPU it runs on
+ * until the process ends; the call makes no hipMalloc / hipFree and uses no allocating library
+ * routine.  Arguments and results are those of tyr_hip_gqa_decode (same kernels).
+ *
+ * Limit: tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits) must not exceed
+ * TYR_HIP_GQA_DECODE_STATIC_SCRATCH_BYTES, else TYR_HIP_ERR_WORKSPACE is returned and nothing is
+ * launched (B * Hq * num_splits <= 16131 at D = 128).
+ * Every call on one GPU uses the same array: calls that overlap in time on one GPU (different
+ * streams, different threads) race on it; calls on one stream are ordered and safe.  Nothing in
+ * the array has to start at zero (the split pass writes every partial the combine pass reads).
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call
+ * outside stream capture.
+ */
+#define TYR_HIP_GQA_DECODE_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+int tyr_hip_gqa_decode_static(const void* q, const void* k, const void* v, void* o, float* lse,
+                              uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                              uint64_t kv_stride, float scale, uint64_t num_splits, void* stream);
+
 /* Flash-attention backward for the forward of tyr_hip_flash_attn_fwd_gqa (same q, k, v, causal,
  * window, kv_lens, scale; o and lse its outputs).  dq : bf16 [B, Hq, N, D]; dk, dv : bf16
  * [B, Hkv, N, D], each summed over the Hq/Hkv query heads that read that kv head (the gradient of

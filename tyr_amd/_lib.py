@@ -14,7 +14,7 @@ SYMBOLS = (
     "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_fwd_gqa", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
     "tyr_hip_flash_attn_bwd_gqa", "tyr_hip_flash_attn_fwd_mask", "tyr_hip_flash_attn_bwd_mask",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
-    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
+    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_fp8",
     "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy",
 )
 
@@ -63,6 +63,8 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_gqa_decode.restype = ci
     L.tyr_hip_gqa_decode_varlen.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, u64, u64, vp, u64, f32, u64, vp, sz, vp]
     L.tyr_hip_gqa_decode_varlen.restype = ci
+    L.tyr_hip_gqa_decode_static.argtypes = [vp, vp, vp, vp, vp, u64, u64, u64, u64, u64, u64, f32, u64, vp]
+    L.tyr_hip_gqa_decode_static.restype = ci
     L.tyr_hip_gemm_bf16.argtypes = [vp, vp, vp, u64, u64, u64, ci, vp]
     L.tyr_hip_gemm_bf16.restype = ci
     L.tyr_hip_gemm_fp8.argtypes = [vp, vp, vp, u64, u64, u64, f32, f32, ci, vp]

@@ -8,6 +8,9 @@
 #include <limits.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "launch.hpp"
 
 namespace {
@@ -33,6 +36,39 @@ uint64_t auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {
 }
 
 }  // namespace
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Partials of the split pass live in a file-scope device array.  Its name is only a host-side
+// stand-in: the address a kernel may use is looked up once per device with hipGetSymbolAddress
+// (every device holds its own copy of the array at its own address) and kept below.
+constexpr size_t kStaticScratchBytes = TYR_HIP_GQA_DECODE_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];            // device address of `scratch`, per device
+static std::atomic<int> g_scratch_state[kMaxDevices];   // 0 = unresolved, 1 = resolved
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return TYR_HIP_ERR_NO_DEVICE;
+    }
+    if (g_scratch_state[dev].load(std::memory_order_acquire) == 0) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_state[dev].load(std::memory_order_relaxed) == 0) {
+            void* ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+                (void)hipGetLastError();
+                return TYR_HIP_ERR_NO_DEVICE;
+            }
+            g_scratch_ptr[dev] = ptr;
+            g_scratch_state[dev].store(1, std::memory_order_release);
+        }
+    }
+    *out = g_scratch_ptr[dev];
+    return TYR_HIP_OK;
+}
 
 extern "C" {
 
@@ -228,6 +264,24 @@ int tyr_hip_gqa_decode_varlen(const void* q, const void* k, const void* v, void*
                                           (int)(window > (uint64_t)INT_MAX ? INT_MAX : window),
                                           static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
+}
+
+int tyr_hip_gqa_decode_static(const void* q, const void* k, const void* v, void* o, float* lse,
+                              uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t L, uint64_t D,
+                              uint64_t kv_stride, float scale, uint64_t num_splits, void* stream) {
+    // sizes are judged before anything touches the device, so an oversized request is an error
+    // return and never a launch
+    if (B == 0 || Hq == 0 || Hkv == 0 || L == 0 || D == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (num_splits > kMaxSplits) return TYR_HIP_ERR_UNSUPPORTED;
+    if (B > (uint64_t)INT_MAX || Hq > (uint64_t)INT_MAX || B * Hq > (uint64_t)INT_MAX || Hkv > Hq || D > 4096)
+        return TYR_HIP_ERR_BAD_SHAPE;
+    const size_t need = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
+    if (need > kStaticScratchBytes) return TYR_HIP_ERR_WORKSPACE;
+    void* ptr = nullptr;
+    const int rc = static_scratch(&ptr);
+    if (rc != TYR_HIP_OK) return rc;
+    return tyr_hip_gqa_decode_varlen(q, k, v, o, lse, B, Hq, Hkv, L, D, kv_stride, nullptr, 0, scale, num_splits,
+                                     ptr, kStaticScratchBytes, stream);
 }
 
 int tyr_hip_decode_rope_append(const void* q, const void* k_new, const void* v_new, const float* cos,
