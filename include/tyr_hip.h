@@ -301,12 +301,28 @@ int tyr_hip_copy(const void* src, void* dst, size_t bytes, void* stream);
  *
  *   a : bf16 [M, K]   b : bf16 [K, N] or [N, K]   c : bf16 [M, N]
  * Supported: M, N, K >= 1 with K % 8 == 0 and N % 8 == 0 (16-byte rows).
- * With TYR_HIP_GEMM_GENERAL set in the environment, this and the fp8 GEMM run their general
- * (register-staged) kernels on every shape; unset, only shapes whose 256-row panels or whose [K, N]
- * B exceed 32-bit byte offsets do.  The switch exists for tests and for comparing the two paths.
  */
 int tyr_hip_gemm_bf16(const void* a, const void* b, void* c,
                       uint64_t M, uint64_t N, uint64_t K, int trans_b, void* stream);
+
+/* Batched form: `batch` independent products C_i = A_i B_i in one launch, entry i at
+ * a + i*stride_a, b + i*stride_b, c + i*stride_c (strides in elements, multiples of 8).
+ * GPU twin of `lean_torch_matmul` (cc/src/tyr.cpp:1565-1570) for operands of rank > 2:
+ * [batch, M, K] x [batch, K, N] with stride_a = M*K, stride_b = K*N, stride_c = M*N, and the
+ * broadcast case [batch, M, K] x [K, N] with stride_b = 0.  batch <= 65535; stride_c >= M*N.
+ * tyr_hip_gemm_bf16 is this call with batch = 1.
+ */
+int tyr_hip_gemm_bf16_batched(const void* a, const void* b, void* c, uint64_t batch,
+                              uint64_t M, uint64_t N, uint64_t K,
+                              uint64_t stride_a, uint64_t stride_b, uint64_t stride_c,
+                              int trans_b, void* stream);
+
+/* Test switch (no counterpart in the reference).  The bf16 and fp8 GEMMs have a fast kernel and a
+ * general (register-staged) kernel that otherwise serves only shapes whose 256-row panels or whose
+ * [K, N] B exceed 32-bit byte offsets.  on != 0 sends every shape through the general kernels,
+ * process-wide, until switched off again; the previous setting is returned.  The initial setting is
+ * "on" iff the environment variable TYR_HIP_GEMM_GENERAL exists when the first GEMM is launched. */
+int tyr_hip_gemm_force_general(int on);
 
 /* ---------------------------------------------------------------------------
  * FP8 E4M3 GEMM with per-tensor f32 scales, bf16 output:
@@ -322,6 +338,19 @@ int tyr_hip_gemm_bf16(const void* a, const void* b, void* c,
 int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c,
                      uint64_t M, uint64_t N, uint64_t K,
                      float scale_a, float scale_b, int trans_b, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Calibration: the MFMA rate this device sustains on the caller's operand bits.
+ *
+ * No counterpart in the reference; it belongs to the measurement side, where the reference's
+ * runners print a torch figure beside the kernel's (Examples/GPU/RunMhaH100Train.lean:217-288).
+ * Every wave of `workgroups` 4-wave workgroups loads 8 operand fragments from `operands` once and
+ * then issues only MFMAs (32x32x16 bf16 or 32x32x64 E4M3), `iters` rounds of 16.  *flop_per_launch
+ * receives the floating-point operations of one launch.  `sink` takes 256 floats per workgroup.
+ */
+enum tyr_hip_mfma_type { TYR_HIP_MFMA_BF16 = 0, TYR_HIP_MFMA_E4M3 = 1 };
+int tyr_hip_mfma_sustain(const void* operands, size_t operand_bytes, int dtype, uint64_t workgroups,
+                         uint64_t iters, float* sink, double* flop_per_launch, void* stream);
 
 #ifdef __cplusplus
 }

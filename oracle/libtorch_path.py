@@ -51,6 +51,17 @@ def sdpa_4d_backward(q, k, v, d_o, is_causal: bool):
     return q32.grad, k32.grad, v32.grad
 
 
+def train_step(q_m, k_m, v_m, target32, lr: float, is_causal: bool = False):
+    """`oneTorchTrainStep` (Examples/GPU/RunMhaH100Train.lean:95-113): f32 SDPA of the detached masters, loss =
+    0.5 mean((out - target)^2), autograd, SGD.  Returns the updated masters and the loss."""
+    ql, kl, vl = (t.detach().requires_grad_(True) for t in (q_m, k_m, v_m))
+    out = F.scaled_dot_product_attention(ql, kl, vl, None, 0.0, is_causal)
+    diff = out - target32
+    loss = (diff * diff).mean() * 0.5
+    loss.backward()
+    return q_m - ql.grad * lr, k_m - kl.grad * lr, v_m - vl.grad * lr, loss.detach()
+
+
 def sdpa_gqa_qkv(q, k, v, is_causal: bool = False, enable_gqa: bool = True, dropout_p: float = 0.0):
     n_head, n_kv_head = q.shape[1], k.shape[1]
     if enable_gqa and n_head != n_kv_head and n_kv_head > 0:

@@ -46,6 +46,12 @@ def test_host_validation_needs_no_gpu():
     assert L.tyr_hip_gemm_bf16(p, p, p, 8, 8, 12, 0, None) == UNSUP
     assert L.tyr_hip_gemm_bf16(p + 2, p, p, 8, 8, 8, 0, None) == MISAL
     assert L.tyr_hip_gemm_bf16(p, p, p, 2 ** 40, 8, 8, 0, None) == SHAPE
+    assert L.tyr_hip_gemm_bf16_batched(p, p, p, 0, 8, 8, 8, 64, 64, 64, 0, None) == SHAPE
+    assert L.tyr_hip_gemm_bf16_batched(p, p, p, 2, 8, 8, 8, 64, 64, 32, 0, None) == SHAPE      # outputs would overlap
+    assert L.tyr_hip_gemm_bf16_batched(p, p, p, 2, 8, 8, 8, 68, 64, 64, 0, None) == MISAL
+    assert L.tyr_hip_gemm_bf16_batched(p, p, p, 70000, 8, 8, 8, 64, 64, 64, 0, None) == SHAPE
+    prev = L.tyr_hip_gemm_force_general(1)
+    assert L.tyr_hip_gemm_force_general(prev) == 1 and L.tyr_hip_gemm_force_general(prev) == prev
     assert L.tyr_hip_gemm_fp8(p, p, None, 16, 16, 16, 1.0, 1.0, 0, None) == NULL
     assert L.tyr_hip_gemm_fp8(p, p, p, 16, 8, 16, 1.0, 1.0, 0, None) == UNSUP
     assert L.tyr_hip_flash_attn_fwd(p, p, None, p, None, 1, 1, 16, 128, 1, 0.1, None) == NULL

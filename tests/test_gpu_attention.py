@@ -334,6 +334,34 @@ def test_gqa_decode_full_size_config(gpu):
     assert torch.equal(gpu.gqa_decode(q, k, v, scale=sc)[0], o)
 
 
+@pytest.mark.parametrize("splits", [2, 4, 8])
+def test_gqa_decode_full_size_config_split_kv_and_combine(gpu, splits):
+    # The same configuration through the two-pass path: split pass writing f32 partials + LSE-combine pass.
+    B, Hq, Hkv, L, D = 32, 32, 8, 8192, 128
+    torch.manual_seed(4)
+    q = torch.randn(B, Hq, 1, D, device="cuda").to(torch.bfloat16)
+    k = torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16)
+    v = torch.randn(B, Hkv, L, D, device="cuda").to(torch.bfloat16)
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.gqa_decode(q, k, v, scale=sc, num_splits=splits)
+    G = Hq // Hkv
+    s = torch.einsum("bkgd,bkld->bkgl", q.view(B, Hkv, G, D).float(), k.float()) * sc
+    ref_lse = torch.logsumexp(s, -1).view(B, Hq)
+    ref = torch.einsum("bkgl,bkld->bkgd", torch.softmax(s, -1), v.float()).reshape(B, Hq, 1, D)
+    assert max_abs(o.float(), ref) <= TOL
+    assert max_abs(lse, ref_lse) <= TOL
+    # three sequences against the scalar C restatement run with the same number of splits
+    for b in (0, 13, 31):
+        wo, wl = oracle.gqa_decode(bits(q[b:b + 1]), bits(k[b:b + 1]), bits(v[b:b + 1]), sc, splits)
+        assert max_abs(o[b:b + 1].cpu().float(), from_bits(wo).float()) <= TOL
+        assert max_abs(lse[b:b + 1].cpu(), wl) <= 1e-3
+    # split-count invariance at full size: one split (single pass) agrees within one bf16 ulp of the outputs
+    o1, lse1 = gpu.gqa_decode(q, k, v, scale=sc, num_splits=1)
+    assert max_abs(o.float(), o1.float()) <= 2.0 ** -7 * float(o1.float().abs().max())
+    assert max_abs(lse, lse1) <= 1e-4
+    assert torch.equal(gpu.gqa_decode(q, k, v, scale=sc, num_splits=splits)[0], o)      # deterministic
+
+
 def test_attention_error_convention(gpu):
     from tyr_amd import TyrGpuError
     q = torch.zeros(1, 1, 16, 128, dtype=torch.bfloat16)

@@ -22,6 +22,16 @@ def gpu():
     return tyr_amd
 
 
+@pytest.fixture
+def general_kernels():
+    """Every GEMM inside the test takes the general (register-staged) kernels."""
+    from tyr_amd import _lib
+    L = _lib.load()
+    prev = L.tyr_hip_gemm_force_general(1)
+    yield
+    assert L.tyr_hip_gemm_force_general(prev) == 1
+
+
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 512, 4096), (8, 8, 8),
                                    (300, 264, 72), (1, 16, 8), (257, 8, 520), (1024, 768, 256), (768, 512, 320),
@@ -74,10 +84,9 @@ def test_gemm_random_shapes(gpu, seed):
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (300, 264, 72), (1, 16, 8), (257, 8, 520)])
-def test_gemm_general_kernels_match_oracle(gpu, monkeypatch, M, N, K, trans_b):
+def test_gemm_general_kernels_match_oracle(gpu, general_kernels, M, N, K, trans_b):
     # The general (register-staged) kernels serve shapes beyond the fast kernels' 32-bit offsets;
-    # the environment switch sends ordinary shapes through them.
-    monkeypatch.setenv("TYR_HIP_GEMM_GENERAL", "1")
+    # the library's switch sends ordinary shapes through them.
     a, b = lt.make_inputs(100 + M + N + K, (M, K), (K, N), std=K ** -0.25)
     bb = b.t().contiguous() if trans_b else b
     c = gpu.gemm_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
@@ -223,3 +232,30 @@ def test_error_convention(gpu):
         gpu.gemm_bf16(a.cuda(), torch.zeros(32, 16, dtype=torch.bfloat16).cuda()[::2])
     with pytest.raises(TyrGpuError, match="not supported"):
         gpu.gemm_bf16(torch.zeros(16, 12, dtype=torch.bfloat16).cuda(), torch.zeros(12, 16, dtype=torch.bfloat16).cuda())
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("shape,broadcast_b", [((3, 300, 264, 72), False), ((2, 5, 64, 128, 256), False),
+                                               ((4, 257, 512, 64), True), ((7, 1, 16, 8), False)])
+def test_batched_matmul_matches_per_entry_gemm_and_libtorch(gpu, shape, broadcast_b, trans_b):
+    # `lean_torch_matmul` on operands of rank > 2 (cc/src/tyr.cpp:1565-1570): one launch for all entries,
+    # bit-identical to the 2-D entry point entry by entry, and within the GEMM bar of torch.matmul in f32.
+    *lead, M, N, K = shape
+    a, = lt.make_inputs(9000 + M + K, (*lead, M, K), std=K ** -0.25)
+    b, = lt.make_inputs(9001 + N + K, ((K, N) if broadcast_b else (*lead, K, N)), std=K ** -0.25)
+    bb = b.transpose(-1, -2).contiguous() if trans_b else b
+    c = gpu.matmul_bf16(a.cuda(), bb.cuda(), trans_b=trans_b).cpu()
+    assert tuple(c.shape) == (*lead, M, N)
+    assert rel_fro(c, torch.matmul(a.float(), b.float())) <= TOL_FRO
+    a2, c2 = a.reshape(-1, M, K), c.reshape(-1, M, N)
+    b2 = None if broadcast_b else bb.reshape(-1, *bb.shape[-2:])
+    for i in range(a2.shape[0]):
+        one = gpu.gemm_bf16(a2[i].cuda(), (bb if broadcast_b else b2[i]).cuda(), trans_b=trans_b).cpu()
+        assert np.array_equal(bits(one), bits(c2[i])), i
+
+
+def test_batched_matmul_through_the_general_kernels(gpu, general_kernels):
+    a, = lt.make_inputs(9100, (3, 130, 72), std=72 ** -0.25)
+    b, = lt.make_inputs(9101, (3, 72, 40), std=72 ** -0.25)
+    c = gpu.matmul_bf16(a.cuda(), b.cuda()).cpu()
+    assert rel_fro(c, torch.matmul(a.float(), b.float())) <= TOL_FRO

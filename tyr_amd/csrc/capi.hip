@@ -8,6 +8,8 @@
 #include <limits.h>
 #include <string.h>
 
+#include <stdlib.h>
+
 #include <atomic>
 #include <mutex>
 
@@ -36,6 +38,26 @@ uint64_t auto_splits(uint64_t B, uint64_t Hkv, uint64_t L) {
 }
 
 }  // namespace
+
+// ---- process-wide switch between the fast and the general GEMM kernels (read on every GEMM launch,
+// so it is an atomic flag; the environment is consulted once, when the flag is first needed)
+namespace tyr {
+static std::atomic<int> g_gemm_general{-1};          // -1 = not initialised
+bool gemm_general_only() {
+    int v = g_gemm_general.load(std::memory_order_relaxed);
+    if (v < 0) {
+        v = getenv("TYR_HIP_GEMM_GENERAL") != nullptr ? 1 : 0;
+        int expected = -1;
+        if (!g_gemm_general.compare_exchange_strong(expected, v)) v = expected;
+    }
+    return v != 0;
+}
+int set_gemm_general_only(int on) {
+    const int prev = gemm_general_only() ? 1 : 0;
+    g_gemm_general.store(on ? 1 : 0);
+    return prev;
+}
+}  // namespace tyr
 
 // ---- the entry point that allocates nothing ---------------------------------------------------
 // Partials of the split pass live in a file-scope device array.  Its name is only a host-side
@@ -343,16 +365,32 @@ int tyr_hip_copy(const void* src, void* dst, size_t bytes, void* stream) {
 
 int tyr_hip_gemm_bf16(const void* a, const void* b, void* c, uint64_t M, uint64_t N, uint64_t K,
                       int trans_b, void* stream) {
+    return tyr_hip_gemm_bf16_batched(a, b, c, 1, M, N, K, 0, 0, 0, trans_b, stream);
+}
+
+int tyr_hip_gemm_bf16_batched(const void* a, const void* b, void* c, uint64_t batch, uint64_t M, uint64_t N,
+                              uint64_t K, uint64_t stride_a, uint64_t stride_b, uint64_t stride_c, int trans_b,
+                              void* stream) {
     if (!a || !b || !c) return TYR_HIP_ERR_NULL_POINTER;
-    if (M == 0 || N == 0 || K == 0) return TYR_HIP_ERR_BAD_SHAPE;
-    if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return TYR_HIP_ERR_BAD_SHAPE;
+    if (batch == 0 || M == 0 || N == 0 || K == 0) return TYR_HIP_ERR_BAD_SHAPE;
+    if (!fits_int(M) || !fits_int(N) || !fits_int(K) || batch > 65535) return TYR_HIP_ERR_BAD_SHAPE;
     if (((M + 255) / 256) * ((N + 255) / 256) > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
     if (K % 8 != 0 || N % 8 != 0) return TYR_HIP_ERR_UNSUPPORTED;
     if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return TYR_HIP_ERR_MISALIGNED;
-    const int rc = tyr::launch_gemm_bf16(a, b, c, (int)M, (int)N, (int)K, trans_b != 0,
+    if (batch > 1) {
+        // every batch entry keeps 16-byte alignment; outputs of different entries must not overlap
+        if (stride_a % 8 != 0 || stride_b % 8 != 0 || stride_c % 8 != 0) return TYR_HIP_ERR_MISALIGNED;
+        if (stride_c < M * N) return TYR_HIP_ERR_BAD_SHAPE;
+        if (stride_a > ((uint64_t)1 << 40) || stride_b > ((uint64_t)1 << 40) || stride_c > ((uint64_t)1 << 40))
+            return TYR_HIP_ERR_BAD_SHAPE;
+    }
+    const int rc = tyr::launch_gemm_bf16(a, b, c, (int)M, (int)N, (int)K, trans_b != 0, (int)batch,
+                                         (int64_t)stride_a, (int64_t)stride_b, (int64_t)stride_c,
                                          static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }
+
+int tyr_hip_gemm_force_general(int on) { return tyr::set_gemm_general_only(on); }
 
 int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c, uint64_t M, uint64_t N, uint64_t K,
                      float scale_a, float scale_b, int trans_b, void* stream) {

@@ -136,8 +136,12 @@ __device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, uint32_t bytes)
 // lds_base + 16 i (lds_base wave-uniform); the source is rsrc.base + voffset + soffset.
 // Issued as opaque asm so that the compiler does not order later LDS reads behind it; the
 // caller waits with wait_vmcnt0() (and a barrier) before anyone reads the destination.  M0 is
-// written here; the compiler keeps nothing live in M0 on this target (it sets M0 itself right
-// before each of its own uses).
+// written here.  M0 is a reserved register for this compiler (it never holds a value across
+// statements; the compiler writes it right before each of its own instructions that read it, and
+// hipcc rejects it on a clobber list with a warning), so the write cannot corrupt compiler state as
+// long as no compiler-generated M0 reader sits between its own write and use -- which
+// tests/test_m0_discipline.py checks on the assembly of every kernel file that includes this one:
+// the only M0 accesses are these writes, each followed by the LDS-DMA loads that consume it.
 __device__ __forceinline__ void load_global_to_lds_16(u32x4 rsrc, uint32_t lds_base, int voffset, int soffset) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"

@@ -16,7 +16,6 @@
 //     multiplied, then written to the other stage: one barrier per slice.
 //   * The MFMA is issued with the B fragment as its row operand, so every lane ends up with
 //     4 consecutive n for one m and stores 8-byte pieces of a C row.
-#include <cstdlib>
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -34,9 +33,13 @@ constexpr int GROUP_M = 4;
 template <bool TRANS_B, bool EDGE>
 __global__ __launch_bounds__(gemm::THREADS) void gemm_bf16_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, int tiles_m, int tiles_n) {
+    int M, int N, int K, int tiles_m, int tiles_n, long stride_a, long stride_b, long stride_c) {
     using namespace gemm;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    // batch entry blockIdx.y (element strides; stride_b = 0 broadcasts one B)
+    A += (size_t)blockIdx.y * stride_a;
+    B += (size_t)blockIdx.y * stride_b;
+    C += (size_t)blockIdx.y * stride_c;
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
@@ -201,9 +204,12 @@ constexpr int GROUP_M = 4;
 template <bool TRANS_B, bool K_TAIL>
 __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, int tiles_m, int tiles_n) {
+    int M, int N, int K, int tiles_m, int tiles_n, long stride_a, long stride_b, long stride_c) {
     using namespace gemm2;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    A += (size_t)blockIdx.y * stride_a;
+    B += (size_t)blockIdx.y * stride_b;
+    C += (size_t)blockIdx.y * stride_c;
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
@@ -377,11 +383,11 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
 }
 
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
-                     hipStream_t stream) {
+                     int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, hipStream_t stream) {
     using namespace gemm;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const bool edge = (M % BM) || (N % BN) || (K % BK);
-    dim3 grid((unsigned)(tiles_m * tiles_n)), block(THREADS);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch), block(THREADS);
     auto A = static_cast<const uint16_t*>(a);
     auto Bp = static_cast<const uint16_t*>(b);
     auto Cp = static_cast<uint16_t*>(c);
@@ -389,9 +395,9 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
     // The fast kernel needs rows of whole 16-byte chunks; ragged M, N and K are handled by the zero
     // fill of the buffer loads (rows past the end, chunks past K) and by the guarded epilogue (columns
     // past N only ever contribute to outputs that are not stored).
-    // TYR_HIP_GEMM_GENERAL (any value) sends every shape to the general kernels, which otherwise only
-    // shapes beyond the 32-bit offsets reach: a switch for tests and for comparing the two paths.
-    const bool general_only = std::getenv("TYR_HIP_GEMM_GENERAL") != nullptr;
+    // gemm_general_only() sends every shape to the general kernels, which otherwise only shapes beyond
+    // the 32-bit offsets reach: a switch for tests and for comparing the two paths.
+    const bool general_only = gemm_general_only();
     const bool fast_ok = !general_only && (K % 8 == 0) && (size_t)256 * K * 2 < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N * 2 < ((size_t)1 << 32));
     if (fast_ok) {
@@ -402,7 +408,8 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm2::LDS_BYTES);                    \
             if (attr != hipSuccess) return -1;                                                    \
             hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB, KT>), grid, block, gemm2::LDS_BYTES, stream, \
-                               A, Bp, Cp, M, N, K, tiles_m, tiles_n);                             \
+                               A, Bp, Cp, M, N, K, tiles_m, tiles_n, (long)stride_a, (long)stride_b,  \
+                               (long)stride_c);                                                   \
         } while (0)
         const bool k_tail = K % gemm2::BK != 0;
         if (trans_b) { if (k_tail) TYR_GEMM_FAST(true, true); else TYR_GEMM_FAST(true, false); }
@@ -417,7 +424,8 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);                               \
         if (attr != hipSuccess) return -1;                                                        \
         hipLaunchKernelGGL((gemm_bf16_kernel<TB, ED>), grid, block, LDS_BYTES, stream, A, Bp, Cp, \
-                           M, N, K, tiles_m, tiles_n);                                            \
+                           M, N, K, tiles_m, tiles_n, (long)stride_a, (long)stride_b,             \
+                           (long)stride_c);                                                       \
     } while (0)
     if (trans_b) { if (edge) TYR_GEMM_LAUNCH(true, true); else TYR_GEMM_LAUNCH(true, false); }
     else         { if (edge) TYR_GEMM_LAUNCH(false, true); else TYR_GEMM_LAUNCH(false, false); }

@@ -11,7 +11,6 @@
 // 128 bytes, k-contiguous padded LDS rows for both operands, two LDS stages with register
 // prefetch, one barrier per slice.  For B stored [K,N] the loader transposes 16(k) x 8(n) byte
 // blocks in registers (two levels of v_perm_b32) on the way to LDS.
-#include <cstdlib>
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -402,9 +401,9 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
     // 32-bit buffer offsets: a 256-row panel of A (and of B^T), or all of B, must stay below 4 GiB
     // The fast kernel needs whole K slices; ragged M and N are handled by the zero fill of the
     // buffer loads and by the guarded epilogue.
-    // TYR_HIP_GEMM_GENERAL (any value) sends every shape to the general kernels, which otherwise only
+    // gemm_general_only() sends every shape to the general kernels, which otherwise only
     // shapes beyond the 32-bit offsets reach: a switch for tests and for comparing the two paths.
-    const bool general_only = std::getenv("TYR_HIP_GEMM_GENERAL") != nullptr;
+    const bool general_only = gemm_general_only();
     const bool fast_ok = !general_only && (K % 16 == 0) && (size_t)256 * K < ((size_t)1 << 31) &&
                          (trans_b || (size_t)K * N < ((size_t)1 << 32));
     if (fast_ok) {

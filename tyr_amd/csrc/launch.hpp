@@ -7,8 +7,14 @@
 
 namespace tyr {
 
+// `batch` independent products; strides in elements between consecutive batch entries (stride_b = 0
+// uses one B for every entry).
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
-                     hipStream_t stream);
+                     int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, hipStream_t stream);
+// Process-wide switch that sends every GEMM shape through the general (register-staged) kernels.
+// Its initial value is taken once from the environment variable TYR_HIP_GEMM_GENERAL.
+bool gemm_general_only();
+int set_gemm_general_only(int on);   // returns the previous value
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
                     int trans_b, hipStream_t stream);
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,

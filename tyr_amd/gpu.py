@@ -278,6 +278,33 @@ def copy(src, stream=None):
     return dst
 
 
+def matmul_bf16(a, b, trans_b: bool = False, stream=None):
+    """C = matmul a b for operands of rank > 2 (`lean_torch_matmul`): a bf16 [..., M, K]; b bf16 [..., K, N] with
+    the same leading extents, or a plain [K, N] matrix used for every batch entry (b is [..., N, K] / [N, K] with
+    trans_b) -> bf16 [..., M, N]."""
+    _check(a, "a", torch.bfloat16)
+    _check(b, "b", torch.bfloat16)
+    if a.dim() < 2 or b.dim() < 2:
+        raise TyrGpuError("a and b must have dim >= 2")
+    if a.dim() == 2 and b.dim() == 2:
+        return gemm_bf16(a, b, trans_b, stream)
+    if b.dim() != 2 and (b.dim() != a.dim() or b.shape[:-2] != a.shape[:-2]):
+        raise TyrGpuError("b must be a matrix or share a's leading extents")
+    if a.dim() == 2:
+        raise TyrGpuError("a must carry the batch extents")
+    M, K = a.shape[-2:]
+    N, Kb = (b.shape[-2], b.shape[-1]) if trans_b else (b.shape[-1], b.shape[-2])
+    if Kb != K:
+        raise TyrGpuError("a and b have mismatched inner dimensions")
+    batch = a.numel() // (M * K) if M * K else 0
+    c = torch.empty(tuple(a.shape[:-2]) + (M, N), dtype=torch.bfloat16, device=a.device)
+    rc = _lib.load().tyr_hip_gemm_bf16_batched(a.data_ptr(), b.data_ptr(), c.data_ptr(), batch, M, N, K, M * K,
+                                               0 if b.dim() == 2 else K * N, M * N, int(bool(trans_b)),
+                                               _stream(stream))
+    _raise(rc, "matmul")
+    return c
+
+
 def gemm_bf16(a, b, trans_b: bool = False, stream=None):
     """C = gemmBf16 a b.  a bf16 [M,K]; b bf16 [K,N] (or [N,K] with trans_b) -> bf16 [M,N]."""
     _check(a, "a", torch.bfloat16, 2)
