@@ -48,3 +48,31 @@ def test_decode_step_replays_from_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(got_o, want_o) and torch.equal(got_lse, want_lse), replay
         assert torch.equal(kg, ke) and torch.equal(vg, ve), replay
+
+
+def test_calls_on_a_side_stream_allocate_on_that_stream():
+    # Outputs and scratch of a call with `stream=` must belong to that stream (the caching allocator reuses a
+    # freed block on the stream it was allocated on): the scratch of a backward or split-decode call queued on a
+    # side stream is dropped at return while its kernels are still pending, and current-stream allocations that
+    # follow must not be handed that block.  Results must equal those of the same calls on the current stream.
+    import tyr_amd
+    B, H, N, D = 2, 4, 600, 128
+    q, k, v, g = (t.cuda() for t in lt.make_inputs(8, (B, H, N, D), (B, H, N, D), (B, H, N, D), (B, H, N, D)))
+    qd, = lt.make_inputs(9, (B, 8, 1, D))
+    kd, vd = (t.cuda() for t in lt.make_inputs(10, (B, 2, 3000, D), (B, 2, 3000, D)))
+    qd = qd.cuda()
+    o, lse = tyr_amd.flash_attn_fwd(q, k, v, causal=True)
+    want = tyr_amd.flash_attn_bwd(q, k, v, o, lse, g, causal=True)
+    want_d = tyr_amd.gqa_decode(qd, kd, vd, num_splits=6)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    for handle in (side, side.cuda_stream):          # a torch stream object and a raw hipStream_t handle
+        got = tyr_amd.flash_attn_bwd(q, k, v, o, lse, g, causal=True, stream=handle)
+        got_d = tyr_amd.gqa_decode(qd, kd, vd, num_splits=6, stream=handle)
+        # churn on the current stream while the side stream is still busy
+        junk = [torch.full((1 << 20,), float(i), device="cuda") for i in range(8)]
+        side.synchronize()
+        for a, b in zip(got + got_d, want + want_d):
+            assert torch.equal(a, b)
+        del junk

@@ -26,6 +26,8 @@
 #ifdef TYR_HAVE_LEAN
 #include <lean/lean.h>
 #include <torch/torch.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <cmath>
 #include <string>
@@ -50,6 +52,20 @@ bool check(const torch::Tensor& t, const char* name, c10::ScalarType dt, std::st
     if (t.scalar_type() != dt) { err = std::string(name) + " has the wrong dtype"; return false; }
     return true;
 }
+
+// Outputs and scratch are allocated by LibTorch's caching allocator, which hands a freed block to
+// the next allocation on the stream it was allocated on.  The kernels run on the caller's `stream`,
+// so for the duration of a call that stream is made LibTorch's current one: the blocks then belong
+// to it, and a scratch tensor dropped at the end of the call (while its kernels are still queued)
+// can only be reused by work queued behind them on the same stream.
+struct LaunchStreamScope {
+    static c10::hip::HIPStreamMasqueradingAsCUDA wrap(uint64_t stream, c10::DeviceIndex dev) {
+        return stream ? c10::hip::getStreamFromExternalMasqueradingAsCUDA(reinterpret_cast<hipStream_t>(stream), dev)
+                      : c10::hip::getDefaultHIPStreamMasqueradingAsCUDA(dev);
+    }
+    c10::hip::HIPStreamGuardMasqueradingAsCUDA guard;
+    LaunchStreamScope(uint64_t stream, const torch::Tensor& like) : guard(wrap(stream, like.device().index())) {}
+};
 
 lean_object* pair_result(torch::Tensor a, torch::Tensor b) {
     lean_object* p = lean_alloc_ctor(0, 2, 0);
@@ -77,6 +93,7 @@ lean_object* lean_tyr_gpu_flash_attn_fwd(uint64_t B, uint64_t H, uint64_t N, uin
         if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
             !check(v_, "v", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto o = torch::empty_like(q_);
         auto lse = torch::empty({(int64_t)B, (int64_t)H, (int64_t)N}, q_.options().dtype(torch::kFloat32));
         const int rc = tyr_hip_flash_attn_fwd(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
@@ -100,11 +117,38 @@ lean_object* lean_tyr_gpu_flash_attn_fwd_gqa(uint64_t B, uint64_t Hq, uint64_t H
         if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
             !check(v_, "v", torch::kBFloat16, err) || !check(n_, "kvLens", torch::kInt32, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto o = torch::empty_like(q_);
         auto lse = torch::empty({(int64_t)B, (int64_t)Hq, (int64_t)N}, q_.options().dtype(torch::kFloat32));
         const int rc = tyr_hip_flash_attn_fwd_gqa(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
                                                   lse.data_ptr<float>(), B, Hq, Hkv, N, D, causal, window,
                                                   n_.data_ptr<int32_t>(), (float)scale, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnFwdGQA", rc);
+        return pair_result(std::move(o), std::move(lse));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// flashAttnFwdGQAFull: flashAttnFwdGQA for sequences that all have N keys (no length tensor, so the launch takes the
+// kernel without the length and window instructions when window = 0).
+// flashAttnFwdGQAFull {B Hq Hkv N D} q k v causal window scale stream : IO (T #[B,Hq,N,D] x T #[B,Hq,N])
+lean_object* lean_tyr_gpu_flash_attn_fwd_gqa_full(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                             b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                             uint8_t causal, uint64_t window, double scale,
+                                             uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err))
+            return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
+        auto o = torch::empty_like(q_);
+        auto lse = torch::empty({(int64_t)B, (int64_t)Hq, (int64_t)N}, q_.options().dtype(torch::kFloat32));
+        const int rc = tyr_hip_flash_attn_fwd_gqa(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
+                                                  lse.data_ptr<float>(), B, Hq, Hkv, N, D, causal, window,
+                                                  nullptr, (float)scale, reinterpret_cast<void*>(stream));
         if (rc != TYR_HIP_OK) return status_error("flashAttnFwdGQA", rc);
         return pair_result(std::move(o), std::move(lse));
     } catch (const std::exception& e) {
@@ -127,6 +171,7 @@ lean_object* lean_tyr_gpu_flash_attn_bwd(uint64_t B, uint64_t H, uint64_t N, uin
             !check(v_, "v", torch::kBFloat16, err) || !check(o_, "o", torch::kBFloat16, err) ||
             !check(g_, "dO", torch::kBFloat16, err) || !check(lse_, "lse", torch::kFloat32, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto dq = torch::empty_like(q_), dk = torch::empty_like(q_), dv = torch::empty_like(q_);
         const size_t ws_bytes = tyr_hip_flash_attn_bwd_workspace_bytes(B, H, N, D);
         auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
@@ -162,6 +207,7 @@ lean_object* lean_tyr_gpu_flash_attn_bwd_gqa(uint64_t B, uint64_t Hq, uint64_t H
             !check(g_, "dO", torch::kBFloat16, err) || !check(lse_, "lse", torch::kFloat32, err) ||
             !check(n_, "kvLens", torch::kInt32, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto dq = torch::empty_like(q_), dk = torch::empty_like(k_), dv = torch::empty_like(k_);
         const size_t ws_bytes = tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D);
         auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
@@ -169,6 +215,42 @@ lean_object* lean_tyr_gpu_flash_attn_bwd_gqa(uint64_t B, uint64_t Hq, uint64_t H
                                                   g_.data_ptr(), lse_.data_ptr<float>(), dq.data_ptr(), dk.data_ptr(),
                                                   dv.data_ptr(), B, Hq, Hkv, N, D, causal, window,
                                                   n_.data_ptr<int32_t>(), (float)scale, ws.data_ptr(), ws_bytes,
+                                                  reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("flashAttnBwdGQA", rc);
+        lean_object* inner = lean_alloc_ctor(0, 2, 0);
+        lean_ctor_set(inner, 0, giveTensor(std::move(dk)));
+        lean_ctor_set(inner, 1, giveTensor(std::move(dv)));
+        lean_object* outer = lean_alloc_ctor(0, 2, 0);
+        lean_ctor_set(outer, 0, giveTensor(std::move(dq)));
+        lean_ctor_set(outer, 1, inner);
+        return lean_io_result_mk_ok(outer);
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// flashAttnBwdGQAFull {B Hq Hkv N D} q k v o lse dO causal window scale stream : IO (dQ x dK x dV)
+lean_object* lean_tyr_gpu_flash_attn_bwd_gqa_full(uint64_t B, uint64_t Hq, uint64_t Hkv, uint64_t N, uint64_t D,
+                                             b_lean_obj_arg q, b_lean_obj_arg k, b_lean_obj_arg v,
+                                             b_lean_obj_arg o, b_lean_obj_arg lse, b_lean_obj_arg d_o,
+                                             uint8_t causal, uint64_t window, double scale,
+                                             uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto q_ = borrowTensor(q), k_ = borrowTensor(k), v_ = borrowTensor(v), o_ = borrowTensor(o);
+        auto lse_ = borrowTensor(lse), g_ = borrowTensor(d_o);
+        std::string err;
+        if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
+            !check(v_, "v", torch::kBFloat16, err) || !check(o_, "o", torch::kBFloat16, err) ||
+            !check(g_, "dO", torch::kBFloat16, err) || !check(lse_, "lse", torch::kFloat32, err))
+            return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
+        auto dq = torch::empty_like(q_), dk = torch::empty_like(k_), dv = torch::empty_like(k_);
+        const size_t ws_bytes = tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D);
+        auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
+        const int rc = tyr_hip_flash_attn_bwd_gqa(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o_.data_ptr(),
+                                                  g_.data_ptr(), lse_.data_ptr<float>(), dq.data_ptr(), dk.data_ptr(),
+                                                  dv.data_ptr(), B, Hq, Hkv, N, D, causal, window,
+                                                  nullptr, (float)scale, ws.data_ptr(), ws_bytes,
                                                   reinterpret_cast<void*>(stream));
         if (rc != TYR_HIP_OK) return status_error("flashAttnBwdGQA", rc);
         lean_object* inner = lean_alloc_ctor(0, 2, 0);
@@ -196,6 +278,7 @@ lean_object* lean_tyr_gpu_flash_attn_fwd_mask(uint64_t B, uint64_t Hq, uint64_t 
             !check(v_, "v", torch::kBFloat16, err) || !check(m_, "keyMask", torch::kUInt8, err))
             return io_error(err);
         if ((uint64_t)m_.numel() != B * N) return io_error("flashAttnFwdMask: keyMask must hold B*N bytes");
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto o = torch::empty_like(q_);
         auto lse = torch::empty({(int64_t)B, (int64_t)Hq, (int64_t)N}, q_.options().dtype(torch::kFloat32));
         const int rc = tyr_hip_flash_attn_fwd_mask(q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr(),
@@ -225,6 +308,7 @@ lean_object* lean_tyr_gpu_flash_attn_bwd_mask(uint64_t B, uint64_t Hq, uint64_t 
             !check(m_, "keyMask", torch::kUInt8, err))
             return io_error(err);
         if ((uint64_t)m_.numel() != B * N) return io_error("flashAttnBwdMask: keyMask must hold B*N bytes");
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto dq = torch::empty_like(q_), dk = torch::empty_like(k_), dv = torch::empty_like(k_);
         const size_t ws_bytes = tyr_hip_flash_attn_bwd_workspace_bytes(B, Hq, N, D);
         auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, q_.options().dtype(torch::kUInt8));
@@ -256,6 +340,7 @@ lean_object* lean_tyr_gpu_gqa_decode(uint64_t B, uint64_t Hq, uint64_t Hkv, uint
         if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
             !check(v_, "v", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto o = torch::empty_like(q_);
         auto lse = torch::empty({(int64_t)B, (int64_t)Hq}, q_.options().dtype(torch::kFloat32));
         const size_t ws_bytes = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
@@ -282,6 +367,7 @@ lean_object* lean_tyr_gpu_gqa_decode_varlen(uint64_t B, uint64_t Hq, uint64_t Hk
         if (!check(q_, "q", torch::kBFloat16, err) || !check(k_, "k", torch::kBFloat16, err) ||
             !check(v_, "v", torch::kBFloat16, err) || !check(n_, "kvLens", torch::kInt32, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto o = torch::empty_like(q_);
         auto lse = torch::empty({(int64_t)B, (int64_t)Hq}, q_.options().dtype(torch::kFloat32));
         const size_t ws_bytes = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
@@ -313,6 +399,7 @@ lean_object* lean_tyr_gpu_decode_rope_append(uint64_t B, uint64_t Hq, uint64_t H
             !check(s_, "sin", torch::kFloat32, err) || !check(kc, "kCache", torch::kBFloat16, err) ||
             !check(vc, "vCache", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, q_);   // outputs and scratch belong to the launch stream
         auto q_out = torch::empty_like(q_);
         const int rc = tyr_hip_decode_rope_append(q_.data_ptr(), kn.data_ptr(), vn.data_ptr(), c_.data_ptr<float>(),
                                                   s_.data_ptr<float>(), q_out.data_ptr(), kc.data_ptr(), vc.data_ptr(),
@@ -334,6 +421,7 @@ lean_object* lean_tyr_gpu_rope_fwd(uint64_t B, uint64_t S, uint64_t H, uint64_t 
         if (!check(x_, "x", bf16 ? torch::kBFloat16 : torch::kFloat32, err) ||
             !check(c_, "cos", torch::kFloat32, err) || !check(s_, "sin", torch::kFloat32, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, x_);   // outputs and scratch belong to the launch stream
         auto y = torch::empty_like(x_);
         const int rc = tyr_hip_rope_fwd(x_.data_ptr(), c_.data_ptr<float>(), s_.data_ptr<float>(), y.data_ptr(), B, S,
                                         H, D, bf16 ? TYR_HIP_BF16 : TYR_HIP_F32, reinterpret_cast<void*>(stream));
@@ -354,6 +442,7 @@ lean_object* lean_tyr_gpu_layernorm_residual(uint64_t rows, uint64_t d, b_lean_o
         if (!check(x_, "x", torch::kBFloat16, err) || !check(r_, "residual", torch::kBFloat16, err) ||
             !check(w_, "weight", torch::kBFloat16, err) || !check(b_, "bias", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, x_);   // outputs and scratch belong to the launch stream
         auto out = torch::empty_like(x_), out_resid = torch::empty_like(x_);
         const int rc = tyr_hip_layernorm_residual(x_.data_ptr(), r_.data_ptr(), w_.data_ptr(), b_.data_ptr(),
                                                   out.data_ptr(), out_resid.data_ptr(), rows, d, (float)eps,
@@ -371,6 +460,7 @@ lean_object* lean_tyr_gpu_copy(lean_obj_arg /*shape*/, b_lean_obj_arg input, uin
         auto in_ = borrowTensor(input);
         if (!in_.is_cuda()) return io_error("input must be a CUDA tensor");
         if (!in_.is_contiguous()) return io_error("input must be contiguous");
+        LaunchStreamScope on_stream(stream, in_);   // outputs and scratch belong to the launch stream
         auto out = torch::empty_like(in_);
         const int rc = tyr_hip_copy(in_.data_ptr(), out.data_ptr(), (size_t)in_.nbytes(), reinterpret_cast<void*>(stream));
         if (rc != TYR_HIP_OK) return status_error("copy", rc);
@@ -388,6 +478,7 @@ lean_object* lean_tyr_gpu_gemm_bf16(uint64_t M, uint64_t N, uint64_t K, b_lean_o
         std::string err;
         if (!check(a_, "a", torch::kBFloat16, err) || !check(b_, "b", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
         auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options());
         const int rc = tyr_hip_gemm_bf16(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, 0,
                                          reinterpret_cast<void*>(stream));
@@ -406,6 +497,7 @@ lean_object* lean_tyr_gpu_gemm_bf16_nt(uint64_t M, uint64_t N, uint64_t K, b_lea
         std::string err;
         if (!check(a_, "a", torch::kBFloat16, err) || !check(b_, "b", torch::kBFloat16, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
         auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options());
         const int rc = tyr_hip_gemm_bf16(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, 1,
                                          reinterpret_cast<void*>(stream));
@@ -425,6 +517,7 @@ lean_object* lean_tyr_gpu_gemm_fp8(uint64_t M, uint64_t N, uint64_t K, b_lean_ob
         std::string err;
         if (!check(a_, "a", torch::kFloat8_e4m3fn, err) || !check(b_, "b", torch::kFloat8_e4m3fn, err))
             return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
         auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options().dtype(torch::kBFloat16));
         const int rc = tyr_hip_gemm_fp8(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, (float)scale_a,
                                         (float)scale_b, 0, reinterpret_cast<void*>(stream));

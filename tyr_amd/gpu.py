@@ -12,6 +12,7 @@ current stream only; all arithmetic happens in ``libtyr_hip.so``.
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
 
 import torch
@@ -56,6 +57,25 @@ def _stream(stream) -> int:
     return int(stream)
 
 
+def _on_launch_stream(fn):
+    """Outputs and scratch come from torch's caching allocator, which ties a block to the stream that was
+    current when it was allocated and may hand a freed block to the next allocation on that stream.  The kernels
+    run on the caller's ``stream``; when that is not torch's current stream it is made current for the call, so the
+    blocks belong to it and a scratch tensor dropped on return (its kernels still queued) can only be reused by
+    work queued behind them.  ``stream`` may be a ``torch.cuda.Stream`` or a raw ``hipStream_t`` handle."""
+    @functools.wraps(fn)
+    def wrapper(*args, stream=None, **kwargs):
+        if stream is None:
+            return fn(*args, stream=None, **kwargs)
+        if isinstance(stream, torch.cuda.Stream):
+            s = stream
+        else:
+            s = torch.cuda.ExternalStream(int(stream)) if int(stream) else torch.cuda.default_stream()
+        with torch.cuda.stream(s):
+            return fn(*args, stream=s.cuda_stream, **kwargs)
+    return wrapper
+
+
 def device_info(device: int = 0) -> dict:
     L = _lib.load()
     name = ctypes.create_string_buffer(64)
@@ -81,6 +101,7 @@ def _key_mask_ptr(key_mask, B, N, window, kv_lens):
     return key_mask.data_ptr()
 
 
+@_on_launch_stream
 def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, window: int = 0, kv_lens=None,
                    key_mask=None, stream=None):
     """O, LSE = flashAttnFwd q k v causal scale.
@@ -121,6 +142,7 @@ def flash_attn_fwd(q, k, v, causal: bool = True, scale: float | None = None, win
     return o, lse
 
 
+@_on_launch_stream
 def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | None = None, window: int = 0,
                    kv_lens=None, key_mask=None, stream=None):
     """dQ, dK, dV = flashAttnBwd q k v o lse dO causal scale.
@@ -168,6 +190,7 @@ def flash_attn_bwd(q, k, v, o, lse, d_o, causal: bool = True, scale: float | Non
     return dq, dk, dv
 
 
+@_on_launch_stream
 def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len: int | None = None,
                kv_lens=None, window: int = 0, stream=None):
     """O, LSE = gqaDecode q k v scale numSplits.
@@ -206,6 +229,7 @@ def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len:
     return o, lse
 
 
+@_on_launch_stream
 def decode_rope_append(q, k_new, v_new, cos, sin, k_cache, v_cache, pos: int, stream=None):
     """qRot = decodeRopeAppend q kNew vNew cos sin kCache vCache pos.
 
@@ -237,6 +261,7 @@ def decode_rope_append(q, k_new, v_new, cos, sin, k_cache, v_cache, pos: int, st
     return q_out
 
 
+@_on_launch_stream
 def rope_fwd(x, cos, sin, stream=None):
     """y = applyRotaryEmb x cos sin.  x f32 or bf16 [B,S,H,D]; cos, sin f32 [S,D/2]."""
     if x.dtype not in (torch.float32, torch.bfloat16):
@@ -254,6 +279,7 @@ def rope_fwd(x, cos, sin, stream=None):
     return y
 
 
+@_on_launch_stream
 def layernorm_residual(x, residual, weight, bias, eps: float = 1e-5, stream=None):
     """(out, outResid) = fusedLayerNormResidual x residual weight bias.  bf16; x, residual [..., d]; weight, bias [d]."""
     for t, n in ((x, "x"), (residual, "residual"), (weight, "weight"), (bias, "bias")):
@@ -269,6 +295,7 @@ def layernorm_residual(x, residual, weight, bias, eps: float = 1e-5, stream=None
     return out, out_resid
 
 
+@_on_launch_stream
 def copy(src, stream=None):
     """out = copy src (any dtype, contiguous)."""
     _check(src, "input", src.dtype)
@@ -278,6 +305,7 @@ def copy(src, stream=None):
     return dst
 
 
+@_on_launch_stream
 def matmul_bf16(a, b, trans_b: bool = False, stream=None):
     """C = matmul a b for operands of rank > 2 (`lean_torch_matmul`): a bf16 [..., M, K]; b bf16 [..., K, N] with
     the same leading extents, or a plain [K, N] matrix used for every batch entry (b is [..., N, K] / [N, K] with
@@ -287,7 +315,7 @@ def matmul_bf16(a, b, trans_b: bool = False, stream=None):
     if a.dim() < 2 or b.dim() < 2:
         raise TyrGpuError("a and b must have dim >= 2")
     if a.dim() == 2 and b.dim() == 2:
-        return gemm_bf16(a, b, trans_b, stream)
+        return gemm_bf16(a, b, trans_b, stream=stream)
     if b.dim() != 2 and (b.dim() != a.dim() or b.shape[:-2] != a.shape[:-2]):
         raise TyrGpuError("b must be a matrix or share a's leading extents")
     if a.dim() == 2:
@@ -305,6 +333,7 @@ def matmul_bf16(a, b, trans_b: bool = False, stream=None):
     return c
 
 
+@_on_launch_stream
 def gemm_bf16(a, b, trans_b: bool = False, stream=None):
     """C = gemmBf16 a b.  a bf16 [M,K]; b bf16 [K,N] (or [N,K] with trans_b) -> bf16 [M,N]."""
     _check(a, "a", torch.bfloat16, 2)
@@ -320,6 +349,7 @@ def gemm_bf16(a, b, trans_b: bool = False, stream=None):
     return c
 
 
+@_on_launch_stream
 def gemm_fp8(aq, bq, scale_a: float, scale_b: float, trans_b: bool = False, stream=None):
     """C = gemmFp8 aq bq scaleA scaleB.  aq e4m3 [M,K]; bq e4m3 [K,N] (or [N,K]) -> bf16 [M,N]."""
     _check(aq, "a", torch.float8_e4m3fn, 2)

@@ -53,6 +53,14 @@ opaque flashAttnFwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : 
     (kvLens : @& T #[B]) (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
     : IO (T #[B, Hq, N, D] × T #[B, Hq, N])
 
+/-- `flashAttnFwdGQA` for a batch whose sequences all have `N` keys: no length tensor, and with `window = 0`
+    the launch takes the kernel instantiation that carries no length or window instructions (the one
+    `flashAttnFwd` runs), which is what a model's ordinary prefill wants (`Tyr/Model/Qwen/Attention.lean:138`). -/
+@[extern "lean_tyr_gpu_flash_attn_fwd_gqa_full"]
+opaque flashAttnFwdGQAFull {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hq, N])
+
 /-- Flash-attention backward. `o` and `lse` are the results of `flashAttnFwd` for the same
     `q k v causal scale`; `dO` is the upstream gradient. Returns `(dQ, dK, dV)`, bf16, final
     (no per-tile partials to reduce on the host). Replaces `tkMhaH100BwdPrep2Block` +
@@ -70,6 +78,13 @@ opaque flashAttnBwd {B H N D : UInt64} (q k v o : @& T #[B, H, N, D]) (lse : @& 
 @[extern "lean_tyr_gpu_flash_attn_bwd_gqa"]
 opaque flashAttnBwdGQA {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
     (o : @& T #[B, Hq, N, D]) (lse : @& T #[B, Hq, N]) (dO : @& T #[B, Hq, N, D]) (kvLens : @& T #[B])
+    (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
+    : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
+
+/-- Backward of `flashAttnFwdGQAFull`. -/
+@[extern "lean_tyr_gpu_flash_attn_bwd_gqa_full"]
+opaque flashAttnBwdGQAFull {B Hq Hkv N D : UInt64} (q : @& T #[B, Hq, N, D]) (k v : @& T #[B, Hkv, N, D])
+    (o : @& T #[B, Hq, N, D]) (lse : @& T #[B, Hq, N]) (dO : @& T #[B, Hq, N, D])
     (causal : Bool) (window : UInt64) (scale : Float) (stream : CudaStream)
     : IO (T #[B, Hq, N, D] × T #[B, Hkv, N, D] × T #[B, Hkv, N, D])
 
