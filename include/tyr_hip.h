@@ -216,7 +216,8 @@ int tyr_hip_flash_attn_bwd_mask(const void* q, const void* k, const void* v, con
  * cc/src/tyr.cpp:3953-4016), the query standing at the last valid position:
  * sequence b attends to cache rows [max(0, len_b - window), len_b), len_b = kv_lens[b].
  *
- *   kv_lens : device int32 [B], each clamped to [1, L]; NULL = every sequence has L rows
+ *   kv_lens : device int32 [B], each clamped to [0, L]; NULL = every sequence has L rows.
+ *             A sequence of length 0 gets O = 0 and LSE = -inf.
  *   window  : 0 = unbounded
  *   L       : upper bound of the lengths (sizes the splits and the workspace)
  * Everything else as tyr_hip_gqa_decode, which is this call with kv_lens = NULL, window = 0.

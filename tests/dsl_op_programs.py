@@ -1,13 +1,13 @@
 """Small tile programs that put every statement the gfx950 emitter lowers through the whole path
-(builder -> emitter -> hipcc -> GPU), one family of statements per program.  They are compiled into
-`libtyr_dsl_ops.so` next to the reference's kernels and exist for the parity tests: each writes the
+(builder -> emitter -> hipcc -> GPU), one family of statements per program.  They are test programs, not part
+of the product: `build()` below compiles them into `tests/build/libtyr_dsl_ops.so` and they exist for the parity tests: each writes the
 result of every operation it covers to its own block of the output, where the test compares it with
 the same operation done by the CPU checker.  The reference tests its lowering one statement at a time
 on text (Tyr/GPU/Codegen/Tests.lean:31-431); these do it on values."""
 from __future__ import annotations
 
-from .builder import KernelBuilder
-from .ir import UNARY_OPS, Kernel
+from tyr_amd.dsl.builder import KernelBuilder
+from tyr_amd.dsl.ir import UNARY_OPS, Kernel
 
 T = 64
 
@@ -20,7 +20,7 @@ def _emit_tile(k, out, stage, tile, row_block, cols_block=None):
     z = k.constIntVal(0)
     r = k.constIntVal(row_block)
     c = z if cols_block is None else k.constIntVal(cols_block)
-    from .builder import RTileCoord
+    from tyr_amd.dsl.builder import RTileCoord
     k.storeGlobal(out, stage, RTileCoord(z, z, r, c))
 
 
@@ -314,3 +314,26 @@ def dslOpsScanAtomic() -> Kernel:
 
 
 ALL = (dslOpsScanAtomic, dslOpsUnary, dslOpsBinary, dslOpsMasks, dslOpsLayout, dslOpsMma, dslOpsControl)
+
+
+# ---- build step (run by __graft_entry__.build(); the tests only load what it built)
+import os as _os
+
+_HERE = _os.path.dirname(_os.path.abspath(__file__))
+SRC_PATH = _os.path.join(_HERE, "build", "tyr_dsl_ops.hip")
+LIB_PATH = _os.path.join(_HERE, "build", "libtyr_dsl_ops.so")
+
+
+def build(lib_path: str = LIB_PATH) -> str:
+    """Emits the programs above as one HIP translation unit and compiles it for gfx950."""
+    from tyr_amd.dsl import build as dsl_build
+    return dsl_build.compile_programs(ALL, SRC_PATH, lib_path)
+
+
+def load():
+    from tyr_amd.dsl import runtime
+    return runtime.load(LIB_PATH)
+
+
+if __name__ == "__main__":
+    print(build())

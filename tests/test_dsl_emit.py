@@ -183,7 +183,8 @@ def test_launcher_validates_on_the_host():
 
 def test_statement_coverage_programs_lower_and_are_built():
     # every statement kind the emitter lowers appears in some program that runs on the GPU tests
-    from tyr_amd.dsl import op_programs, runtime
+    from tests import dsl_op_programs as op_programs
+    from tyr_amd.dsl import runtime
     from tyr_amd.dsl.emit import NO_OPS, NVIDIA_ONLY
     used = set()
     for f in kernels.ALL + op_programs.ALL:
@@ -192,7 +193,7 @@ def test_statement_coverage_programs_lower_and_are_built():
         used |= {s.op for s in walk(k.body)}
     lowered = set(KSTMT_FIELDS) - NVIDIA_ONLY - NO_OPS
     assert lowered - used == set(), lowered - used
-    L = runtime.load_op_programs()
+    L = op_programs.load()
     for f in op_programs.ALL:
         assert hasattr(L, f"tyr_launch_{f().name}")
 

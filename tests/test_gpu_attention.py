@@ -334,6 +334,44 @@ def test_gqa_decode_full_size_config(gpu):
     assert torch.equal(gpu.gqa_decode(q, k, v, scale=sc)[0], o)
 
 
+@pytest.mark.parametrize("splits", [0, 1, 4])
+def test_gqa_decode_empty_sequences(gpu, splits):
+    # A sequence whose cache length is 0 attends to nothing: O = 0, LSE = -inf (the convention of the masked
+    # prefill for a row without visible keys); its neighbours are unaffected.
+    B, Hq, Hkv, Lmax, D = 4, 8, 2, 900, 128
+    lens = [0, 900, 0, 17]
+    q, = lt.make_inputs(950, (B, Hq, 1, D))
+    k, v = lt.make_inputs(951, (B, Hkv, Lmax, D), (B, Hkv, Lmax, D))
+    sc = 1 / math.sqrt(D)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    o, lse = gpu.gqa_decode(q.cuda(), k.cuda(), v.cuda(), scale=sc, num_splits=splits, kv_lens=lens_d)
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert torch.count_nonzero(o[b].float()) == 0 and torch.all(torch.isneginf(lse[b]))
+        else:
+            wo, wl = oracle.gqa_decode(bits(q[b:b + 1]), bits(k[b:b + 1, :, :n].contiguous()), bits(v[b:b + 1, :, :n].contiguous()), sc, 1)
+            assert max_abs(o[b:b + 1].cpu().float(), from_bits(wo).float()) <= TOL
+            assert max_abs(lse[b:b + 1].cpu(), wl) <= 1e-3
+
+
+def test_gqa_decode_more_than_65535_groups(gpu):
+    # (batch, kv head) groups are folded into a one-dimensional grid: their number is not limited by grid.y.
+    B, Hq, Hkv, L, D = 8200, 8, 8, 40, 64
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn(B, Hq, 1, D, device="cuda", generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, L, D, device="cuda", generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, L, D, device="cuda", generator=g).to(torch.bfloat16)
+    sc = 1 / math.sqrt(D)
+    o, lse = gpu.gqa_decode(q, k, v, scale=sc)
+    s = torch.einsum("bhd,bhld->bhl", q[:, :, 0].float(), k.float()) * sc
+    ref = torch.einsum("bhl,bhld->bhd", torch.softmax(s, -1), v.float())
+    assert max_abs(o[:, :, 0].float(), ref) <= TOL
+    assert max_abs(lse, torch.logsumexp(s, -1)) <= TOL
+    for b in (0, 8191, 8199):        # both sides of the old limit, against the scalar C restatement
+        wo, wl = oracle.gqa_decode(bits(q[b:b + 1]), bits(k[b:b + 1]), bits(v[b:b + 1]), sc, 1)
+        assert max_abs(o[b:b + 1].cpu().float(), from_bits(wo).float()) <= TOL
+
+
 @pytest.mark.parametrize("splits", [2, 4, 8])
 def test_gqa_decode_full_size_config_split_kv_and_combine(gpu, splits):
     # The same configuration through the two-pass path: split pass writing f32 partials + LSE-combine pass.

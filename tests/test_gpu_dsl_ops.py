@@ -1,4 +1,4 @@
-"""Every statement the gfx950 emitter lowers, on values: the programs of tyr_amd/dsl/op_programs.py run
+"""Every statement the gfx950 emitter lowers, on values: the programs of tests/dsl_op_programs.py run
 on the GPU and each block of their output is compared with the same operation computed on the CPU in
 float32 (float64 for the products).  Bars: exact for data movement, masks, layout changes, comparisons,
 min/max and the bf16 round trip; a few ulp (rtol 2e-5) for arithmetic and transcendental functions,
@@ -13,8 +13,9 @@ T = 64
 
 @pytest.fixture(scope="module")
 def rt():
-    from tyr_amd.dsl import op_programs, runtime
-    return op_programs, runtime, runtime.load_op_programs()
+    from tests import dsl_op_programs as op_programs
+    from tyr_amd.dsl import runtime
+    return op_programs, runtime, op_programs.load()
 
 
 def close(got, want, exact=False):

@@ -273,11 +273,11 @@ int tyr_hip_gqa_decode_varlen(const void* q, const void* k, const void* v, void*
     if (Hq % Hkv != 0 || kv_stride < L) return TYR_HIP_ERR_BAD_SHAPE;
     if ((D != 128 && D != 64) || Hq / Hkv > 16 || num_splits > kMaxSplits) return TYR_HIP_ERR_UNSUPPORTED;
     if (!(scale > 0.0f) || scale > 3.0e38f) return TYR_HIP_ERR_UNSUPPORTED;
-    if (!fits_int(L) || !fits_int(B * Hq) || B * Hkv > 65535 || kv_stride > (uint64_t)INT_MAX)
-        return TYR_HIP_ERR_BAD_SHAPE;
+    if (!fits_int(L) || !fits_int(B * Hq) || kv_stride > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TYR_HIP_ERR_MISALIGNED;
     if (kv_lens && (reinterpret_cast<uintptr_t>(kv_lens) & 3u)) return TYR_HIP_ERR_MISALIGNED;
     if (num_splits == 0) num_splits = auto_splits(B, Hkv, window > 0 && window < L ? window : L);
+    if (!fits_int(B * Hkv * num_splits)) return TYR_HIP_ERR_BAD_SHAPE;      // one workgroup per (group, split)
     const size_t need = tyr_hip_gqa_decode_workspace_bytes(B, Hq, Hkv, L, D, num_splits);
     if (!workspace || workspace_bytes < need) return TYR_HIP_ERR_WORKSPACE;
     if (!aligned16(workspace)) return TYR_HIP_ERR_MISALIGNED;

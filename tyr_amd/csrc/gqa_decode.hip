@@ -9,7 +9,7 @@
 // partial results are merged with the online-softmax algebra
 //   m = max m_s ; l = sum l_s 2^(m_s-m) ; O = sum O_s 2^(m_s-m) / l ; LSE = ln l + m ln 2.
 //
-// First pass.  grid = (splits, B*Hkv), 8 waves per workgroup; the waves take the 32-row steps of
+// First pass.  grid = splits * B*Hkv workgroups (the splits of a group adjacent), 8 waves per workgroup; the waves take the 32-row steps of
 // the split in turn, each with the 16x16x32 bf16 MFMA:
 //   S^T (16 kv x 16 q)  = K rows (row operand: lane l holds row l%16, 8 d at 32i + 8(l/16))
 //                         x Q^T (column operand, zero beyond the G = Hq/Hkv real heads)
@@ -55,16 +55,17 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int x = lane & 15, g = lane >> 4;
-    const int split = blockIdx.x;
-    const int bg = blockIdx.y;                  // b * Hkv + kv head
+    // one-dimensional grid, the splits of a (batch, kv head) group adjacent: any number of groups fits
+    const int split = (int)(blockIdx.x % (unsigned)S);
+    const int bg = (int)(blockIdx.x / (unsigned)S);   // b * Hkv + kv head
     const int b = bg / Hkv, kvh = bg % Hkv;
 
     const uint16_t* Kb = Kp + (size_t)bg * kv_stride * D;
     const uint16_t* Vb = Vp + (size_t)bg * kv_stride * D;
 
     // Per-sequence length (a padding mask over the cache tail) and sliding window: this sequence
-    // attends to cache rows [lo, L).
-    if (kv_lens != nullptr) L = max(1, min(L, kv_lens[b]));
+    // attends to cache rows [lo, L).  A length of zero (an empty sequence) gives O = 0, LSE = -inf.
+    if (kv_lens != nullptr) L = max(0, min(L, kv_lens[b]));
     const int lo = window > 0 ? max(0, L - window) : 0;
     const int c0 = lo + split * chunk;
     const int c1 = min(L, c0 + chunk);
@@ -207,8 +208,8 @@ __global__ __launch_bounds__(64 * WAVES) void gqa_decode_split_kernel(
         }
         const size_t head = (size_t)b * Hq + (size_t)kvh * G + qh;
         if (S == 1) {
-            O[head * D + d] = (uint16_t)(pack_bf16(o / l, 0.0f) & 0xffffu);
-            if (d == 0 && LSE != nullptr) LSE[head] = logf(l) + m * LN2;
+            O[head * D + d] = (uint16_t)(pack_bf16(l > 0.0f ? o / l : 0.0f, 0.0f) & 0xffffu);
+            if (d == 0 && LSE != nullptr) LSE[head] = l > 0.0f ? logf(l) + m * LN2 : -INFINITY;
         } else {
             const size_t ph = head * S + split;
             part_o[ph * D + d] = o;
@@ -242,11 +243,11 @@ __global__ __launch_bounds__(D) void gqa_decode_combine_kernel(
         o += live ? os * wgt : 0.0f;
         l += live ? ls * wgt : 0.0f;
     }
-    const float res = o / l;
+    const float res = l > 0.0f ? o / l : 0.0f;    // every split empty: the sequence has no keys
     // pairs of threads pack two bf16 into one dword
     const float nb = __shfl_down(res, 1);
     if ((d & 1) == 0) reinterpret_cast<uint32_t*>(O + (size_t)bh * D)[d >> 1] = pack_bf16(res, nb);
-    if (LSE != nullptr && d == 0) LSE[bh] = logf(l) + m * LN2;
+    if (LSE != nullptr && d == 0) LSE[bh] = l > 0.0f ? logf(l) + m * LN2 : -INFINITY;
 }
 
 int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, float* lse, int B,
@@ -265,7 +266,7 @@ int launch_gqa_decode(const void* q, const void* k, const void* v, void* o, floa
     float* part_l = part_m + (size_t)B * Hq * S;
 
     const size_t lds = (size_t)(WAVES * G * D + 2 * WAVES * QPAD) * sizeof(float);
-    dim3 grid((unsigned)S, (unsigned)(B * Hkv)), block(64 * WAVES);
+    dim3 grid((unsigned)((size_t)S * B * Hkv)), block(64 * WAVES);
 #define TYR_DEC_LAUNCH(DD)                                                                           \
     do {                                                                                             \
         static const hipError_t attr = hipFuncSetAttribute(                                          \

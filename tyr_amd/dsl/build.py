@@ -6,7 +6,7 @@ from __future__ import annotations
 import os
 import subprocess
 
-from . import kernels, op_programs
+from . import kernels
 from .emit import emit_header, emit_translation_unit
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -14,9 +14,6 @@ CSRC = os.path.join(_PKG, "csrc")
 GEN_DIR = os.path.join(CSRC, "build", "dsl")
 SRC_PATH = os.path.join(GEN_DIR, "tyr_dsl_kernels.hip")
 LIB_PATH = os.path.join(_PKG, "lib", "libtyr_dsl.so")
-# the statement-coverage programs of op_programs.py, used by the tests only
-OPS_SRC_PATH = os.path.join(GEN_DIR, "tyr_dsl_ops.hip")
-OPS_LIB_PATH = os.path.join(_PKG, "lib", "libtyr_dsl_ops.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
             "-packed-fp32-ops"]
@@ -50,8 +47,9 @@ def build(lib_path: str = LIB_PATH) -> str:
     return _compile(emit_sources(), lib_path)
 
 
-def build_op_programs(lib_path: str = OPS_LIB_PATH) -> str:
-    return _compile(emit_sources(OPS_SRC_PATH, op_programs.ALL), lib_path)
+def compile_programs(programs, src_path: str, lib_path: str) -> str:
+    """Emits any list of tile programs (functions returning a Kernel) to `src_path` and compiles it to `lib_path`."""
+    return _compile(emit_sources(src_path, programs), lib_path)
 
 
 if __name__ == "__main__":
@@ -59,4 +57,3 @@ if __name__ == "__main__":
         f.write(header_text())
     print(HEADER_PATH)
     print(build())
-    print(build_op_programs())

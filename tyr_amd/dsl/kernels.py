@@ -1,5 +1,9 @@
 """The reference's end-to-end tested tile programs, written against `KernelBuilder`.
 
+These are input programs, not product logic: each is a statement-for-statement restatement of a Lean
+`@[gpu_kernel]` definition (names and tile shapes included), because the task of the emitter is to run
+those very programs on gfx950.  The product logic is the emitter and the tile library they are lowered by.
+
 Each function builds the same statement sequence as the Lean definition it cites; together they
 are the kernels the reference ships runners for (Examples/GPU/Run{Copy,Rotary,LayerNorm,FlashAttn}.lean)
 plus its canonical GEMM example.

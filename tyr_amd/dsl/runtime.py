@@ -7,7 +7,7 @@ from __future__ import annotations
 import ctypes
 import os
 
-from .build import LIB_PATH, OPS_LIB_PATH
+from .build import LIB_PATH
 from .ir import Kernel
 
 _libs = {}
@@ -23,10 +23,6 @@ def load(path: str = LIB_PATH) -> ctypes.CDLL:
                                "Emitted kernels have no CPU fallback.")
         _libs[path] = ctypes.CDLL(path)
     return _libs[path]
-
-
-def load_op_programs() -> ctypes.CDLL:
-    return load(OPS_LIB_PATH)
 
 
 def launch(kernel: Kernel, args, grid=(1, 1, 1), block=(128, 1, 1), shared_mem: int = 0, stream=None,

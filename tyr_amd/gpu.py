@@ -197,7 +197,7 @@ def gqa_decode(q, k, v, scale: float | None = None, num_splits: int = 0, kv_len:
 
     q bf16 [B,Hq,1,D]; k, v bf16 [B,Hkv,Lmax,D] (the preallocated cache); the first ``kv_len``
     rows (default all) of every (batch, kv head) are attended to.  ``kv_lens`` (int32 [B] on the device)
-    gives every sequence its own length <= kv_len; ``window`` > 0 restricts each sequence to its last
+    gives every sequence its own length in [0, kv_len] (a length of 0 yields O = 0, LSE = -inf); ``window`` > 0 restricts each sequence to its last
     ``window`` rows.  -> (bf16 [B,Hq,1,D], f32 [B,Hq]).
     """
     for t, n in ((q, "q"), (k, "k"), (v, "v")):
