@@ -272,3 +272,56 @@ def test_lds_tiles_with_disjoint_live_ranges_share_storage():
     # sharing would need a barrier the program does not have (the attention forward's Q and K tiles)
     assert "tyr_lds_pool" not in dsl.emit_kernel(kernels.tkFusedLayerNormResidual1024())
     assert "tyr_lds_pool" not in dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())
+
+
+def test_programs_too_large_for_one_wave_are_run_by_a_wave_group():
+    """The H100 bf16 GEMM surface (Bf16Gemm.lean:64-73: a 128x256 f32 accumulator) and the load-compute-finish
+    attention surfaces (MhaH100LCF.lean:84-132: 128x128 / 192x64 K and V tiles beside a 64 x D accumulator) do not fit
+    one wave's registers.  The emitter keeps their B operands in LDS and cuts the row-tied tiles into per-wave row
+    slices; programs that fit one wave are emitted as before."""
+    from tyr_amd.dsl.emit import _Emitter, peak_tile_registers, wave_group_plan, infer_rv_layouts, REG_BUDGET
+    for f in kernels.ALL:
+        k = f()
+        w, split, streamed = wave_group_plan(k, infer_rv_layouts(k))
+        if k.name in ("tkH100Bf16GemmFwd", "tkMhaH100LCFFwd64", "tkMhaH100LCFFwd128"):
+            assert peak_tile_registers(k) > 512                      # more than a lane's whole register file
+            assert w == (4 if k.name == "tkH100Bf16GemmFwd" else 2)
+            assert peak_tile_registers(k, split, w, set(streamed)) <= REG_BUDGET
+            assert len(streamed) == (1 if k.name == "tkH100Bf16GemmFwd" else 2)
+        else:
+            assert (w, split, streamed) == (1, set(), {}), k.name
+    g = kernels.tkH100Bf16GemmFwd()
+    text = dsl.emit_kernel(g)
+    assert "__launch_bounds__(256)" in text and "const int tyr_wave = wave::index();" in text
+    assert "rt<float, 32, 256, layout::row>" in text and "rt<float, 128, 256" not in text
+    assert "wave::load_part(" in text and "wave::store_part(" in text and ", tyr_wave * 32);" in text
+    assert re.search(r"wave::mma_ABt\(v\d+, v\d+, v14, v\d+\);", text)           # B operand = the LDS tile itself
+    # a row slice stored to LDS is followed by a barrier before the group reads the whole tile
+    i = text.index("wave::store(v17")
+    assert text[i:].split("\n")[1].strip().startswith("wave::sync();")
+    # the launcher takes exactly the group's wave count
+    assert "if (waves != 4) return -2;" in _Emitter(g).launcher_text()
+    a = dsl.emit_kernel(kernels.tkMhaH100LCFFwd128())
+    assert "rt<float, 32, 128, layout::row>" in a and a.count("stays in LDS") == 2
+    assert re.search(r"rv<float, 32, vlayout::align>", a)                         # per-row softmax state is sliced too
+
+
+def test_operands_that_cannot_stay_in_lds_keep_their_registers():
+    from tyr_amd.dsl.emit import streamed_operands
+    # the backward program uses K both as a product's A operand and in a layout swap: it must stay a register tile
+    assert streamed_operands(kernels.tkMhaH100Bwd2BlockPartials()) == {}
+    # a tile whose LDS source is overwritten between its load and its product must not be streamed
+    k = dsl.KernelBuilder("overwritten")
+    p = k.gptr("BFloat16", "p")
+    coord = k.blockCoord2D()
+    a, b = k.allocRT("BFloat16", 64, 64), k.allocRT("BFloat16", 64, 64)
+    acc = k.zeroRT("Float32", 64, 64)
+    sa, sb = k.allocST("BFloat16", 64, 64), k.allocST("BFloat16", 64, 64)
+    k.loadGlobal(sa, p, coord)
+    k.loadGlobal(sb, p, coord)
+    k.sync()
+    k.load(a, sa)
+    k.load(b, sb)
+    k.loadGlobal(sb, p, coord.withRow(coord.c))      # sb changes before b is multiplied
+    k.mmaT(acc, a, b, acc)
+    assert streamed_operands(k.build()) == {}

@@ -10,7 +10,7 @@ import torch
 
 import oracle
 from oracle import libtorch_path as lt
-from tests.util import bits, from_bits
+from tests.util import bits, from_bits, max_abs
 
 pytestmark = pytest.mark.gpu
 
@@ -151,6 +151,81 @@ def test_mha_h100_forward_prep_and_backward_programs(rt):
     assert close(dQ, T(want_dq)) and close(dK, T(want_dk)) and close(dV, T(want_dv))
     for got, want in ((dQ.cpu(), T(want_dq)), (dK, T(want_dk)), (dV, T(want_dv))):
         assert float((got.double() - want.double()).norm() / want.double().norm()) <= 1e-2
+
+
+def test_mha_h100_seq768_forward_prep_and_backward_programs(rt):
+    """Examples/GPU/RunMhaH100Seq768.lean:100-136 on q, k, v, dO [1,1,768,64]: the 12-block forwards, the prep
+    program and the 12-block backward with its dK / dV partials summed over the 12 query tiles on the host, at the
+    runner's bars (allclose 5e-2 forward, 8e-2 backward) and at a relative Frobenius error of 1e-2."""
+    kernels, runtime = rt
+    q, k, v, dO = lt.make_inputs(23, (1, 1, 768, 64), (1, 1, 768, 64), (1, 1, 768, 64), (1, 1, 768, 64))
+    geo = dict(grid=(1, 12, 1), block=(128, 1, 1))
+    qc, kc, vc, dOc = (t.cuda() for t in (q, k, v, dO))
+    out_lse, lse = torch.zeros_like(qc), torch.zeros(12, 64).cuda()
+    runtime.launch(kernels.tkFlashAttnFwd12BlockLse(), [qc, kc, vc, out_lse, lse, 768, 64], **geo)
+    out_plain = torch.zeros_like(qc)
+    runtime.launch(kernels.tkFlashAttnFwd12Block(), [qc, kc, vc, out_plain, 768, 64], **geo)
+    out, l_out = torch.zeros_like(qc), torch.zeros(12, 64).cuda()
+    runtime.launch(kernels.tkMhaH100Fwd12Block(), [qc, kc, vc, out, l_out, 768, 64], **geo)
+    d_vec = torch.zeros(12, 64).cuda()
+    runtime.launch(kernels.tkMhaH100BwdPrep2Block(), [dOc, out, d_vec, 768, 64], **geo)
+    dQ = torch.zeros(1, 1, 768, 64).cuda()
+    dK_part, dV_part = torch.zeros(1, 1, 768, 768).cuda(), torch.zeros(1, 1, 768, 768).cuda()
+    runtime.launch(kernels.tkMhaH100Bwd12BlockPartials(), [qc, kc, vc, dOc, l_out, d_vec, dQ, dK_part, dV_part, 768, 64],
+                   **geo)
+    torch.cuda.synchronize()
+    dK = dK_part.reshape(1, 1, 12, 64, 12, 64).sum(4).reshape(1, 1, 768, 64).cpu()
+    dV = dV_part.reshape(1, 1, 12, 64, 12, 64).sum(4).reshape(1, 1, 768, 64).cpu()
+    want_o, want_lse = oracle.attn_fwd_f64(bits(q), bits(k), bits(v), False, 0.125)
+    want_dq, want_dk, want_dv = oracle.attn_bwd_f64(bits(q), bits(k), bits(v), bits(dO), False, 0.125)
+    T = torch.from_numpy
+    close = lambda a, b, tol: torch.allclose(a.cpu().float(), b.float(), rtol=tol, atol=tol)
+    assert torch.equal(out, out_lse) and torch.equal(out, out_plain)
+    assert close(out, T(want_o), 5e-2) and close(out, T(want_o), 2e-2)
+    assert close(l_out.reshape(768), -8.0 * T(want_lse).reshape(768), 5e-2)
+    assert torch.allclose(l_out, -8.0 * lse, rtol=0, atol=1e-4)
+    assert close(dQ, T(want_dq), 8e-2) and close(dK, T(want_dk), 8e-2) and close(dV, T(want_dv), 8e-2)
+    for got, want in ((dQ.cpu(), T(want_dq)), (dK, T(want_dk)), (dV, T(want_dv))):
+        assert float((got.double() - want.double()).norm() / want.double().norm()) <= 1e-2
+
+
+@pytest.mark.parametrize("name,D", [("tkMhaH100LCFFwd64", 64), ("tkMhaH100LCFFwd128", 128)])
+def test_mha_h100_lcf_forward_programs(rt, name, D):
+    """Tyr/GPU/Kernels/MhaH100LCF.lean:84-132: a stationary 64 x D query tile against 3072 streamed keys (16 tiles of
+    192 rows at D = 64, 24 tiles of 128 rows at D = 128), non-causal.  The program is run by a group of two waves
+    (64 threads of the reference = 2 warps), K and V staying in LDS.  Checked against softmax(Q K^T scale) V in
+    float64 on the same bf16 inputs at the attention bar."""
+    kernels, runtime = rt
+    nq, nkv = 192, 3072
+    q, k, v = lt.make_inputs(41 + D, (1, 1, nq, D), (1, 1, nkv, D), (1, 1, nkv, D))
+    o = torch.zeros(1, 1, nq, D, dtype=torch.bfloat16).cuda()
+    runtime.launch(getattr(kernels, name)(), [q.cuda(), k.cuda(), v.cuda(), o, nkv, D], grid=(1, nq // 64, 1), block=(64, 1, 1))
+    torch.cuda.synchronize()
+    sc = 0.125 if D == 64 else 0.08838834764
+    p = torch.softmax(q[0, 0].double() @ k[0, 0].double().T * sc, -1)
+    want = p @ v[0, 0].double()
+    assert max_abs(o[0, 0].cpu().float(), want) <= 2e-2
+    assert float((o[0, 0].cpu().double() - want).norm() / want.norm()) <= 1e-2
+    # any other block size is refused: the compiled program is a group of exactly two waves
+    with pytest.raises(RuntimeError, match="invalid launch arguments"):
+        runtime.launch(getattr(kernels, name)(), [q.cuda(), k.cuda(), v.cuda(), o, nkv, D], grid=(1, 1, 1), block=(128, 1, 1))
+
+
+@pytest.mark.parametrize("M,N", [(128, 256), (384, 1024)])
+def test_tkH100Bf16GemmFwd(rt, M, N):
+    """Tyr/GPU/Kernels/Bf16Gemm.lean:64-73: C[128 x 256 tiles] = A[M, 256] B[N, 256]^T, f32 accumulate, bf16 out; the
+    128 x 256 accumulator is held by a group of four waves (32 rows each), B is read from LDS by the products."""
+    kernels, runtime = rt
+    K = 256                                                  # 4 slices of 64, fixed by the program
+    a, b = lt.make_inputs(51, (M, K), (N, K), std=K ** -0.25)
+    c = torch.zeros(M, N, dtype=torch.bfloat16).cuda()
+    runtime.launch(kernels.tkH100Bf16GemmFwd(), [a.cuda(), b.cuda(), c, M, N, K], grid=(N // 256, M // 128, 1),
+                   block=(128, 1, 1))
+    torch.cuda.synchronize()
+    want = from_bits(oracle.gemm_bf16(bits(a), bits(b), trans_b=True)).float()
+    got = c.cpu().float()
+    assert float((got - a.float() @ b.float().T).norm() / (a.float() @ b.float().T).norm()) <= 1e-2
+    assert (got - want).abs().max() <= 2.0 ** -7 * want.abs().max()
 
 
 def _fp8_inputs(seed, M, N, K):

@@ -729,6 +729,131 @@ __device__ __forceinline__ void col_scan(rt<T, R, C, layout::row>& dst, const rt
 
 __device__ __forceinline__ void sync() { __syncthreads(); }
 
+// ---------------------------------------------------------------- wave groups
+// A program whose register tiles do not fit one wave is run by a group of W waves: tiles and ALIGN
+// vectors that are tied to one another through their rows are cut into W row slices, wave w owning
+// rows [w R/W, (w+1) R/W); everything else (B operands, ORTHO vectors) is common to the group.  The
+// pieces below are what the emitter prints for such a program.
+__device__ __forceinline__ int index() { return (int)(threadIdx.x >> 6); }
+
+// global <-> LDS, the group sharing the tile: wave `part` of `nparts` moves its share of the rows
+template <typename T, int R, int C>
+__device__ __forceinline__ void load_part(st<T, R, C>& dst, const gl<T>& src, coord at, int part, int nparts) {
+    constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
+    static_assert(C % VEC == 0, "rows are whole 16-byte pieces");
+    for (int idx = part * 64 + lane(); idx < R * CPR; idx += 64 * nparts) {
+        const int r = idx / CPR, c = (idx % CPR) * VEC;
+        *reinterpret_cast<u32x4*>(dst.at(r, c)) = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
+    }
+    wave_fence();
+}
+template <typename T, int R, int C>
+__device__ __forceinline__ void store_part(const gl<T>& dst, const st<T, R, C>& src, coord at, int part, int nparts) {
+    constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
+    static_assert(C % VEC == 0, "rows are whole 16-byte pieces");
+    wave_fence();
+    for (int idx = part * 64 + lane(); idx < R * CPR; idx += 64 * nparts) {
+        const int r = idx / CPR, c = (idx % CPR) * VEC;
+        *reinterpret_cast<u32x4*>(dst.at(at.b, at.d, at.r + r, at.c + c)) = *reinterpret_cast<const u32x4*>(src.at(r, c));
+    }
+}
+// a wave's row slice of an LDS tile / vector <-> registers
+template <typename T, int RS, int R, int C>
+__device__ __forceinline__ void load(rt<T, RS, C, layout::row>& dst, const st<T, R, C>& src, int row0) {
+    typedef rt<T, RS, C, layout::row> RT;
+    static_assert(RS <= R, "a slice is no taller than its tile");
+    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *src.at(row0 + row_of<layout::row>(rb, s), col_of<layout::row>(cb, s));
+}
+template <typename T, int RS, int R, int C>
+__device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
+    typedef rt<T, RS, C, layout::row> RT;
+    static_assert(RS <= R, "a slice is no taller than its tile");
+    TYR_TILE_FOR_BLOCKS(RT) *dst.at(row0 + row_of<layout::row>(rb, s), col_of<layout::row>(cb, s)) = src.data[rb][cb][s];
+    wave_fence();
+}
+template <typename T, int NS, int N>
+__device__ __forceinline__ void load(rv<T, NS, vlayout::align>& dst, const sv<T, N>& src, int off) {
+#pragma unroll
+    for (int b = 0; b < NS / 32; ++b) dst.data[b][0] = src.data[off + 32 * b + lr()];
+}
+template <typename T, int NS, int N>
+__device__ __forceinline__ void store(sv<T, N>& dst, const rv<T, NS, vlayout::align>& src, int off) {
+#pragma unroll
+    for (int b = 0; b < NS / 32; ++b)
+        if (lg() == 0) dst.data[off + 32 * b + lr()] = src.data[b][0];
+    wave_fence();
+}
+
+// Products whose B operand stays in LDS: its fragments are read as the product consumes them instead of
+// occupying a register tile (a 256x64 bf16 B would be 256 registers per lane).  The k <-> (lane half,
+// slot) map is that of the register tiles: slot e of half h of lane half g is k = 16h + 8(e/4) + 4g + e%4.
+// B as [N, K] rows (the DSL's mmaT): two 8-byte reads per fragment.
+template <int M, int N, int K>
+__device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<bf16, M, K, layout::row>& a,
+                                        const st<bf16, N, K>& b, const rt<float, M, N, layout::row>& c) {
+#pragma unroll
+    for (int nb = 0; nb < N / 32; ++nb) {
+        f32x16 acc[M / 32];
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+#pragma unroll
+        for (int kb = 0; kb < K / 32; ++kb)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const bf16* p = b.at(32 * nb + lr(), 32 * kb + 16 * h + 4 * lg());
+                const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p), hi = *reinterpret_cast<const bf16x4*>(p + 8);
+                const bf16x8 fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int mb = 0; mb < M / 32; ++mb) {
+                    bf16x8 fa;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
+                    acc[mb] = mfma_32x32x16_bf16(fb, fa, acc[mb]);
+                }
+            }
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+    }
+}
+// B as [K, N] rows in LDS (the DSL's mma with a COL register tile): transposing reads, as load(rt col, st).
+template <int M, int N, int K>
+__device__ __forceinline__ void mma_AB(rt<float, M, N, layout::row>& d, const rt<bf16, M, K, layout::row>& a,
+                                       const st<bf16, K, N>& b, const rt<float, M, N, layout::row>& c) {
+    const int i16 = lane() & 15, b16 = lane() >> 4;
+    const int srow = 4 * (b16 >> 1) + (i16 >> 2), scol = 16 * (b16 & 1) + 4 * (i16 & 3);
+#pragma unroll
+    for (int nb = 0; nb < N / 32; ++nb) {
+        f32x16 acc[M / 32];
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+#pragma unroll
+        for (int kb = 0; kb < K / 32; ++kb)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const bf16x4 lo = ds_read_tr16(b.at(32 * kb + 16 * h + srow, 32 * nb + scol));
+                const bf16x4 hi = ds_read_tr16(b.at(32 * kb + 16 * h + 8 + srow, 32 * nb + scol));
+                const bf16x8 fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int mb = 0; mb < M / 32; ++mb) {
+                    bf16x8 fa;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
+                    acc[mb] = mfma_32x32x16_bf16(fb, fa, acc[mb]);
+                }
+            }
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+    }
+}
+
 }  // namespace wave
 }  // namespace tile
 }  // namespace tyr

@@ -204,7 +204,7 @@ def _lds_regions(kernel: Kernel, plan: Dict[VarId, int]) -> Dict[VarId, Any]:
     return {v: ("lds", find(v).ident) for v in vs}
 
 
-def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None) -> set:
+def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None, streamed: Dict[VarId, VarId] = None) -> set:
     """ids of the statements that need a workgroup barrier in front of them.
 
     Every wave of a workgroup runs the whole tile program, so the LDS tiles and vectors are shared
@@ -222,7 +222,13 @@ def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None) -> 
     def obj(v):
         return {regions.get(v, v)} if v in shared else set()
 
+    streamed = streamed or {}
+
     def rw(s: Stmt):
+        if s.op == "load" and s.dst in streamed:
+            return (set(), set())                        # not read here: the products read the LDS tile themselves
+        if s.op == "mma" and s.b in streamed:
+            return (obj(streamed[s.b]), set())
         if s.op == "load":
             return (obj(s.src), set())
         if s.op == "store":
@@ -274,26 +280,228 @@ def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None) -> 
     return marks
 
 
+# ---------------------------------------------------------------------------- wave groups
+# A program written for one warp of the reference can declare register tiles that no single wave holds
+# (the H100 GEMM surface accumulates 128x256 in f32: 512 registers per lane; the D = 128 attention surface
+# keeps 128x128 K and V tiles next to a 64x128 accumulator).  Such a program is run by a group of W waves:
+#   * B operands that are only loaded from an LDS tile and multiplied stay in LDS ("streamed": the
+#     product reads its fragments as it goes);
+#   * register tiles and per-row vectors that are tied to an accumulator through their rows are cut
+#     into W row slices, one per wave; loads and stores against LDS take the wave's row offset;
+#   * global <-> LDS moves are shared out among the waves.
+REG_BUDGET = 400          # registers per lane a plan may need for its register tiles (of 512)
+
+
+def _rt_regs(d: Stmt, rows=None) -> int:
+    return (rows if rows is not None else d.rows) * d.cols // 64      # one register per element per lane
+
+
+def streamed_operands(kernel: Kernel) -> Dict[VarId, VarId]:
+    """register tile -> LDS tile, for tiles that are defined only by `load` from LDS and used only as the B
+    operand of products in the same statement list, with no write to that LDS tile in between."""
+    info = {s.v: s for s in walk(kernel.body) if s.op in ("declRT", "declST")}
+    uses: Dict[VarId, List[Stmt]] = {}
+    for s in walk(kernel.body):
+        if s.op in ("declRT", "forLoop", "forLoopVal", "ifStmt", "comment"):
+            continue
+        for a in s.args:
+            if isinstance(a, VarId) and a in info and info[a].op == "declRT":
+                uses.setdefault(a, []).append(s)
+    cand = {}
+    for v, us in uses.items():
+        d = info[v]
+        if d.dtype != "BFloat16":
+            continue
+        ok = True
+        for u in us:
+            if u.op == "load" and u.dst == v and u.src in info and info[u.src].op == "declST":
+                continue
+            if u.op == "mma" and u.b == v and v not in (u.dst, u.a, u.c) and (
+                    (u.trans == "ABt" and d.layout == "Row") or (u.trans == "AB" and d.layout == "Col")):
+                continue
+            ok = False
+        if ok and any(u.op == "load" for u in us) and any(u.op == "mma" for u in us):
+            cand[v] = None
+
+    def scan(body):
+        cur: Dict[VarId, VarId] = {}                     # tile -> LDS tile it currently mirrors
+        for s in body:
+            if s.op in ("forLoop", "forLoopVal"):
+                scan(s.body)
+                cur = {}
+            elif s.op == "ifStmt":
+                scan(s.thenBody)
+                scan(s.elseBody)
+                cur = {}
+            elif s.op == "load" and s.dst in cand:
+                cur[s.dst] = s.src
+                if cand[s.dst] not in (None, s.src):
+                    cand[s.dst] = False                  # mirrors two different LDS tiles: keep it in registers
+                elif cand[s.dst] is None:
+                    cand[s.dst] = s.src
+            elif s.op == "mma" and s.b in cand:
+                if s.b not in cur:
+                    cand[s.b] = False                    # multiplied in another statement list than it is loaded in
+            elif s.op in ("loadGlobal", "store"):
+                # LDS tile overwritten: a later product of a tile that mirrors it would see the new data,
+                # so that tile loses its mirror (and a product that follows disqualifies it above)
+                for v in [v for v, st_ in cur.items() if st_ == s.dst]:
+                    del cur[v]
+    scan(kernel.body)
+    return {v: st_ for v, st_ in cand.items() if st_}
+
+
+def row_split_set(kernel: Kernel, rv_layout: Dict[VarId, str], streamed: Dict[VarId, VarId]):
+    """Register tiles and vectors tied to a product's accumulator through their rows, or None when a
+    statement touching them has no row-sliced form."""
+    info = {s.v: s for s in walk(kernel.body) if s.op in ("declRT", "declRV")}
+    parent = {v: v for v in info}
+
+    def find(v):
+        while parent[v] != v:
+            parent[v] = parent[parent[v]]
+            v = parent[v]
+        return v
+
+    def tie(*vs):
+        vs = [v for v in vs if v in info]
+        for v in vs[1:]:
+            parent[find(v)] = find(vs[0])
+
+    seeds = []
+    for s in walk(kernel.body):
+        if s.op == "mma" and s.trans in ("AB", "ABt"):
+            tie(s.dst, s.a, s.c)
+            seeds.append(s.dst)
+        elif s.op == "mm" and s.trans in ("AB", "ABt"):
+            tie(s.dst, s.a)
+            seeds.append(s.dst)
+        elif s.op in ("unary", "convert", "scalarMul", "scalarAdd"):
+            tie(s.dst, s.src)
+        elif s.op == "binary":
+            tie(s.dst, s.a, s.b)
+        elif s.op == "ternary":
+            tie(s.dst, s.a, s.b, s.c)
+        elif s.op == "binaryBroadcast":
+            tie(s.dst, s.tile, *( [s.vec] if s.axis == "Col" else [] ))
+        elif s.op == "broadcast" and s.axis == "Col":
+            tie(s.dst, s.vec)
+        elif s.op == "reduce" and s.axis == "Row":
+            tie(s.dst, s.src)
+        elif s.op == "reduceAccum" and s.axis == "Row":
+            tie(s.dst, s.src, s.accum)
+    roots = {find(v) for v in seeds}
+    split = {v for v in info if find(v) in roots}
+    if not split:
+        return None
+    plain = {"declRT", "declRV", "load", "store", "unary", "convert", "scalarMul", "scalarAdd", "binary", "ternary",
+             "vecFillScalar", "comment"}
+    for s in walk(kernel.body):
+        touched = [a for a in s.args if isinstance(a, VarId) and a in split]
+        if not touched or s.op in plain:
+            continue
+        if s.op in ("mma", "mm"):
+            if s.trans not in ("AB", "ABt") or s.b in split:
+                return None
+        elif s.op == "binaryBroadcast":
+            if s.axis == "Row" and s.vec in split:
+                return None
+        elif s.op == "broadcast":
+            if s.axis != "Col":
+                return None
+        elif s.op in ("reduce", "reduceAccum"):
+            if s.axis != "Row":
+                return None
+        else:
+            return None                                  # masks, transposes, slices, scans ... have no sliced form yet
+    for v in split:
+        d = info[v]
+        if d.op == "declRV" and rv_layout.get(v) != "align":
+            return None
+        if d.op == "declRT" and d.layout != "Row":
+            return None
+    return split
+
+
+def peak_tile_registers(kernel: Kernel, split=frozenset(), waves: int = 1, streamed=frozenset()) -> int:
+    """Most registers per lane the register tiles live at one point need (a tile lives from its first to its
+    last mention; a mention inside a loop counts for the whole loop)."""
+    decl = {s.v: s for s in walk(kernel.body) if s.op == "declRT"}
+    live: Dict[VarId, List[int]] = {}
+    pos = [0]
+
+    def run(body):
+        for s in body:
+            pos[0] += 1
+            if s.op in ("forLoop", "forLoopVal"):
+                start = pos[0]
+                before = {v: list(r) for v, r in live.items()}
+                run(s.body)
+                for v, r in live.items():
+                    if before.get(v) != r and v in before:        # defined outside, used inside: live for the loop
+                        r[0], r[1] = min(r[0], start), max(r[1], pos[0])
+            elif s.op == "ifStmt":
+                run(s.thenBody)
+                run(s.elseBody)
+            elif s.op != "declRT":
+                for a in s.args:
+                    if isinstance(a, VarId) and a in decl and a not in streamed:
+                        r = live.setdefault(a, [pos[0], pos[0]])
+                        r[1] = pos[0]
+    run(kernel.body)
+    peak = 0
+    for p_ in range(1, pos[0] + 1):
+        need = sum(_rt_regs(decl[v], decl[v].rows // waves if v in split else None) for v, r in live.items() if r[0] <= p_ <= r[1])
+        peak = max(peak, need)
+    return peak
+
+
+def wave_group_plan(kernel: Kernel, rv_layout: Dict[VarId, str]):
+    """(waves, split set, streamed map) for a program: (1, {}, {}) when one wave holds it."""
+    if peak_tile_registers(kernel) <= REG_BUDGET:
+        return 1, set(), {}
+    streamed = streamed_operands(kernel)
+    if streamed and peak_tile_registers(kernel, streamed=set(streamed)) <= REG_BUDGET:
+        return 1, set(), streamed
+    split = row_split_set(kernel, rv_layout, streamed)
+    if split:
+        decl = {s.v: s for s in walk(kernel.body) if s.op in ("declRT", "declRV")}
+        for w in (2, 4):
+            sizes = [(decl[v].rows if decl[v].op == "declRT" else decl[v].len) for v in split]
+            if any(n % (32 * w) for n in sizes):
+                continue
+            if peak_tile_registers(kernel, split, w, set(streamed)) <= REG_BUDGET:
+                return w, split, streamed
+    return 1, set(), {}
+
+
 class _Emitter:
     def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True,
-                 prefetch_global_loads: bool = True, share_lds: bool = True):
+                 prefetch_global_loads: bool = True, share_lds: bool = True, wave_group=None):
         self.k = kernel
-        # request the next iteration's global tiles of a loop before the work of the current one
-        self.prefetch_global_loads = prefetch_global_loads
-        # LDS tiles with disjoint live ranges share storage
-        # (only where that asks for no barrier the program does not already have)
-        self.lds = lds_plan(kernel) if share_lds else {}
-        if self.lds and shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds)) != shared_hazard_barriers(kernel):
-            self.lds = {}
-        self.barrier_before = shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds)) if hazard_barriers else set()
-        # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
-        # full 512-register file, and covers the 128-thread blocks the reference's runners launch
-        self.max_waves = max_waves
         self.info: Dict[VarId, Stmt] = {}
         for s in walk(kernel.body):
             if s.op in ("declRT", "declST", "declRV", "declSV", "declGPtr", "declKVal"):
                 self.info[s.v] = s
         self.rv_layout = infer_rv_layouts(kernel)
+        # one wave, or a group of waves sharing the program's tiles (see wave_group_plan)
+        self.waves, self.split, self.streamed = wave_group if wave_group is not None else wave_group_plan(kernel, self.rv_layout)
+        self.group = self.waves > 1
+        self.dirty: set = set()          # LDS objects written in shares by the group since the last barrier
+        # request the next iteration's global tiles of a loop before the work of the current one
+        self.prefetch_global_loads = prefetch_global_loads and not self.group and not self.streamed
+        # LDS tiles with disjoint live ranges share storage
+        # (only where that asks for no barrier the program does not already have)
+        self.lds = lds_plan(kernel) if share_lds else {}
+        if self.lds and shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds), self.streamed) != \
+                shared_hazard_barriers(kernel, None, self.streamed):
+            self.lds = {}
+        self.barrier_before = shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds), self.streamed) \
+            if hazard_barriers else set()
+        # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
+        # full 512-register file, and covers the 128-thread blocks the reference's runners launch.
+        # A wave group needs exactly its own number of waves.
+        self.max_waves = self.waves if self.group else max_waves
 
     def kind(self, v: VarId) -> str:
         s = self.info.get(v)
@@ -310,14 +518,18 @@ class _Emitter:
         if op in NO_OPS:
             return f"{ind}// {op}: nothing to do, an MFMA result is complete when it is read\n"
         if op == "declRT":
-            return f"{ind}rt<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)};\n"
+            if s.v in self.streamed:
+                return f"{ind}// {I(s.v)} stays in LDS: products read their fragments from {I(self.streamed[s.v])}\n"
+            rows = s.rows // self.waves if s.v in self.split else s.rows
+            return f"{ind}rt<{_cpp_type(s.dtype)}, {rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)};\n"
         if op == "declST":
             ty = f"st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}>"
             if s.v in self.lds:
                 return f"{ind}{ty}& {I(s.v)} = *reinterpret_cast<{ty}*>(tyr_lds_pool + {self.lds[s.v]});\n"
             return f"{ind}__shared__ {ty} {I(s.v)};\n"
         if op == "declRV":
-            return f"{ind}rv<{_cpp_type(s.dtype)}, {s.len}, vlayout::{self.rv_layout[s.v]}> {I(s.v)};\n"
+            n = s.len // self.waves if s.v in self.split else s.len
+            return f"{ind}rv<{_cpp_type(s.dtype)}, {n}, vlayout::{self.rv_layout[s.v]}> {I(s.v)};\n"
         if op == "declSV":
             return f"{ind}__shared__ sv<{_cpp_type(s.dtype)}, {s.len}> {I(s.v)};\n"
         if op == "declGPtr":
@@ -325,10 +537,20 @@ class _Emitter:
         if op == "declKVal":
             return f"{ind}// param: {s.name} ({I(s.v)})\n"
         if op in ("load", "store"):
+            reg = s.dst if op == "load" else s.src
+            if reg in self.streamed:
+                return f"{ind}// load of {I(reg)} elided: it stays in {I(self.streamed[reg])}\n"
+            if reg in self.split:                        # this wave's row slice
+                d = self.info[reg]
+                n = (d.rows if d.op == "declRT" else d.len) // self.waves
+                return f"{ind}wave::{op}({I(s.dst)}, {I(s.src)}, tyr_wave * {n});\n"
             return f"{ind}wave::{op}({I(s.dst)}, {I(s.src)});\n"
         if op in ("loadGlobal", "storeGlobal"):
             tile = self.info[s.dst if op == "loadGlobal" else s.src]
             at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)} * {tile.rows}, (int){I(s.coordC)} * {tile.cols}}}"
+            if self.group:                               # the group shares the move
+                return (f"{ind}wave::{'load_part' if op == 'loadGlobal' else 'store_part'}({I(s.dst)}, {I(s.src)}, {at}, "
+                        f"tyr_wave, {self.waves});\n")
             return f"{ind}wave::{'load' if op == 'loadGlobal' else 'store'}({I(s.dst)}, {I(s.src)}, {at});\n"
         if op in ("loadVecGlobal", "storeVecGlobal"):
             return f"{ind}wave::{'load' if op == 'loadVecGlobal' else 'store'}({I(s.dst)}, {I(s.src)}, (int){I(s.offset)});\n"
@@ -356,7 +578,8 @@ class _Emitter:
         if op == "layoutDim":
             return f"{ind}const int {I(s.dst)} = {I(s.src)}.{s.axis.lower()}();\n"
         if op == "mma":
-            return f"{ind}wave::mma_{s.trans}({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.c)});\n"
+            b = self.streamed.get(s.b, s.b)              # a streamed operand is read from its LDS tile
+            return f"{ind}wave::mma_{s.trans}({I(s.dst)}, {I(s.a)}, {I(b)}, {I(s.c)});\n"
         if op == "mm":
             return (f"{ind}wave::unary<op_zero>({I(s.dst)}, {I(s.dst)});\n"
                     f"{ind}wave::mma_{s.trans}({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.dst)});\n")
@@ -419,6 +642,14 @@ class _Emitter:
             pre = self.prefetchable(s) if self.prefetch_global_loads else []
             if pre:
                 return self.prefetched_loop(s, hi, pre, ind)
+            if self.group:                               # what the back edge may bring in, to a fixed point
+                entry = set(self.dirty)
+                while True:
+                    end = self._dirty_after(s.body, entry) | entry
+                    if end == entry:
+                        break
+                    entry = end
+                self.dirty = set(entry)
             return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < {hi}; ++{I(s.v)}) {{\n" + self.body(s.body, ind + "  ") +
                     f"{ind}}}\n")
         if op == "ifStmt":
@@ -531,8 +762,65 @@ class _Emitter:
         for s in stmts:
             if id(s) in self.barrier_before:
                 out += f"{ind}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
-            out += self.stmt(s, ind)
+                self.dirty = set()
+            if self.group:
+                reads, writes = self._group_rw(s)
+                if reads & self.dirty:
+                    out += f"{ind}wave::sync();  // inserted: the other waves' shares of a shared tile are read below\n"
+                    self.dirty = set()
+                if s.op == "sync":
+                    self.dirty = set()
+                out += self.stmt(s, ind)
+                if s.op not in ("forLoop", "forLoopVal", "ifStmt"):
+                    self.dirty |= writes
+            else:
+                out += self.stmt(s, ind)
         return out
+
+    # ------------------------------------------------------------------ wave groups: who reads whose share
+    def _group_rw(self, s: Stmt):
+        """(LDS objects the statement reads in full, LDS objects it leaves written in per-wave shares)."""
+        if s.op in ("forLoop", "forLoopVal"):
+            return set(), set()                          # handled when the loop is emitted
+        if s.op == "ifStmt":                             # a barrier cannot sit inside a conditional
+            r, w = set(), set()
+            for t in walk(s.thenBody + s.elseBody):
+                a, b = self._group_rw(t)
+                r |= a
+                w |= b
+            return r, w
+        if s.op == "load":
+            return (set() if s.dst in self.streamed else {s.src}), set()
+        if s.op == "store":
+            return set(), ({s.dst} if s.src in self.split else set())
+        if s.op == "loadGlobal":
+            return set(), {s.dst}
+        if s.op in ("storeGlobal", "storeGlobalAdd", "storeVecGlobal", "storeVecGlobalCoord", "storeVecGlobalAdd",
+                    "storeVecGlobalAddCoord"):
+            return {s.src}, set()
+        if s.op == "mma" and s.b in self.streamed:
+            return {self.streamed[s.b]}, set()
+        return set(), set()
+
+    def _dirty_after(self, stmts, dirty: set) -> set:
+        dirty = set(dirty)
+        for s in stmts:
+            if id(s) in self.barrier_before or s.op == "sync":
+                dirty = set()
+            if s.op in ("forLoop", "forLoopVal"):
+                entry = set(dirty)
+                while True:
+                    end = self._dirty_after(s.body, entry) | entry
+                    if end == entry:
+                        break
+                    entry = end
+                dirty = self._dirty_after(s.body, entry)
+                continue
+            reads, writes = self._group_rw(s)
+            if reads & dirty:
+                dirty = set()
+            dirty |= writes
+        return dirty
 
     # ------------------------------------------------------------------ kernel + launchers
     def param_decls(self):
@@ -557,7 +845,12 @@ class _Emitter:
                         for v, off in self.lds.items())
             pool = (f"  // LDS tiles whose live ranges do not intersect share these bytes\n"
                     f"  __shared__ __attribute__((aligned(16))) unsigned char tyr_lds_pool[{total}];\n")
-        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" + pool +
+        head = ""
+        if self.group:
+            head = (f"  // run by a group of {self.waves} waves: row-tied register tiles are cut into {self.waves} row slices\n"
+                    f"  const int tyr_wave = wave::index();\n")
+        self.dirty = set()
+        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" + pool + head +
                 self.body(self.k.body, "  ") + "}\n")
 
     def launcher_signature(self) -> str:
@@ -595,8 +888,9 @@ class _Emitter:
             f"extern \"C\" int tyr_launch_{name}({', '.join(cparams)}) {{\n" + "".join(setup) +
             f"  const uint64_t threads = block_x * block_y * block_z;\n"
             f"  if (threads == 0 || grid_x * grid_y * grid_z == 0) return -2;\n"
-            f"  const unsigned waves = (unsigned)((threads + 31) / 32);\n"
-            f"  if (waves > {self.max_waves}) return -2;\n"
+            f"  const unsigned waves = (unsigned)((threads + 31) / 32);\n" +
+            (f"  if (waves != {self.waves}) return -2;   // the program is compiled for a group of exactly {self.waves} waves\n"
+             if self.group else f"  if (waves > {self.max_waves}) return -2;\n") +
             f"  hipLaunchKernelGGL({name}, dim3((unsigned)grid_x, (unsigned)grid_y, (unsigned)grid_z), dim3(64 * waves), "
             f"(size_t)shared_mem, static_cast<hipStream_t>(stream), {', '.join(args)});\n"
             f"  return hipGetLastError() == hipSuccess ? 0 : -1;\n}}\n")

@@ -227,7 +227,7 @@ def simpleGemm(numKBlocks: int = 8) -> Kernel:
     return k.build()
 
 
-def _flash_attn_fwd_2block(name: str, out_kind: str) -> Kernel:
+def _flash_attn_fwd_2block(name: str, out_kind: str, numKvBlocks: int = 2) -> Kernel:
     """The three 2-block forward programs of Tyr/GPU/Kernels/MhaH100.lean share everything but their
     second output: none (`tkFlashAttnFwd2Block`, :14-68), LSE = ln(l) + m (`tkFlashAttnFwd2BlockLse`,
     :71-128) or L = -8 LSE, the ThunderKittens convention for D = 64 (`tkMhaH100Fwd2Block`, :130-190)."""
@@ -240,7 +240,6 @@ def _flash_attn_fwd_2block(name: str, out_kind: str) -> Kernel:
     k.kval("UInt64", "_seq_len")
     k.kval("UInt64", "_head_dim")
     tileSize = 64
-    numKvBlocks = 2
     scale = 0.125
 
     coord = k.blockCoord2D()
@@ -308,6 +307,21 @@ def tkMhaH100Fwd2Block() -> Kernel:
     return _flash_attn_fwd_2block("tkMhaH100Fwd2Block", "l")
 
 
+def tkFlashAttnFwd12Block() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:347-398 -- the same program over 12 KV blocks (seq = 768)."""
+    return _flash_attn_fwd_2block("tkFlashAttnFwd12Block", "none", 12)
+
+
+def tkFlashAttnFwd12BlockLse() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:400-457."""
+    return _flash_attn_fwd_2block("tkFlashAttnFwd12BlockLse", "lse", 12)
+
+
+def tkMhaH100Fwd12Block() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:459-519."""
+    return _flash_attn_fwd_2block("tkMhaH100Fwd12Block", "l", 12)
+
+
 def tkMhaH100BwdPrep2Block() -> Kernel:
     """Tyr/GPU/Kernels/MhaH100.lean:192-227 -- d[row] = sum_j dO[row, j] * O[row, j]."""
     k = KernelBuilder("tkMhaH100BwdPrep2Block")
@@ -346,11 +360,11 @@ def tkMhaH100BwdPrep2Block() -> Kernel:
     return k.build()
 
 
-def tkMhaH100Bwd2BlockPartials() -> Kernel:
+def tkMhaH100Bwd2BlockPartials(name: str = "tkMhaH100Bwd2BlockPartials", numKvBlocks: int = 2) -> Kernel:
     """Tyr/GPU/Kernels/MhaH100.lean:229-344 -- backward of one 64-row query tile over two KV blocks
     (non-causal): dQ final, dK / dV as one 64x64 partial per (kv tile, q tile) that the caller sums
     over q tiles (Examples/GPU/RunMhaH100.lean:131-138).  Scores are kept in K x Q orientation."""
-    k = KernelBuilder("tkMhaH100Bwd2BlockPartials")
+    k = KernelBuilder(name)
     q_ptr = k.gptr("BFloat16", "q_ptr")
     k_ptr = k.gptr("BFloat16", "k_ptr")
     v_ptr = k.gptr("BFloat16", "v_ptr")
@@ -363,7 +377,6 @@ def tkMhaH100Bwd2BlockPartials() -> Kernel:
     k.kval("UInt64", "_seq_len")
     k.kval("UInt64", "_head_dim")
     tileSize = 64
-    numKvBlocks = 2
     scale = 0.125
     invLScale = -0.125
 
@@ -460,6 +473,103 @@ def tkMhaH100Bwd2BlockPartials() -> Kernel:
     return k.build()
 
 
+def tkMhaH100Bwd12BlockPartials() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100.lean:521-640 -- the backward program over 12 KV blocks (seq = 768)."""
+    return tkMhaH100Bwd2BlockPartials("tkMhaH100Bwd12BlockPartials", 12)
+
+
+def _mhaH100LcfFwd(name: str, headDim: int, kvTileRows: int, numKvTiles: int, banner: str, scale: float) -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100LCF.lean:29-82 -- one stationary 64 x D query tile, KV streamed in tiles of
+    kvTileRows rows, online softmax across the stream."""
+    k = KernelBuilder(name)
+    q_ptr = k.gptr("BFloat16", "q_ptr")
+    k_ptr = k.gptr("BFloat16", "k_ptr")
+    v_ptr = k.gptr("BFloat16", "v_ptr")
+    o_ptr = k.gptr("BFloat16", "o_ptr")
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    k.comment(banner)
+    k.comment("ThunderKittens lcf pipeline compressed into a typed single-query-tile shell")
+    k.comment("The exact multi-worker CTA packing is still flattened to one logical query tile per kernel instance.")
+
+    coord = k.blockCoord2D()
+
+    qShared = k.allocST("BFloat16", 64, headDim)
+    kShared = k.allocST("BFloat16", kvTileRows, headDim)
+    vShared = k.allocST("BFloat16", kvTileRows, headDim, "Col")
+    oShared = k.allocST("BFloat16", 64, headDim)
+
+    q = k.allocRT("BFloat16", 64, headDim)
+    kt = k.allocRT("BFloat16", kvTileRows, headDim)
+    v = k.allocRT("BFloat16", kvTileRows, headDim, "Col")
+    o = k.zeroRT("Float32", 64, headDim)
+    softmaxState = k.allocSoftmaxState("Float32", 64)
+
+    k.loadGlobal(qShared, q_ptr, coord)
+    k.sync()
+    k.load(q, qShared)
+
+    with k.krange(0, numKvTiles) as kvIdx:
+        kvCoord = coord.withRow(kvIdx.id)
+        scores = k.zeroRT("Float32", 64, kvTileRows)
+        probs = k.allocRT("BFloat16", 64, kvTileRows)
+
+        k.loadGlobal(kShared, k_ptr, kvCoord)
+        k.loadGlobal(vShared, v_ptr, kvCoord)
+        k.sync()
+        k.load(kt, kShared)
+        k.load(v, vShared)
+
+        k.mmaT(scores, q, kt, scores)
+        k.scalarMul(scores, scores, scale)
+        k.onlineSoftmax(scores, o, softmaxState)
+        k.convert(probs, scores)
+        k.mma(o, probs, v, o)
+        k.sync()
+
+    k.finalizeSoftmax(o, softmaxState)
+    oBf16 = k.allocRT("BFloat16", 64, headDim)
+    k.convert(oBf16, o)
+    k.store(oShared, oBf16)
+    k.storeGlobal(o_ptr, oShared, coord)
+    return k.build()
+
+
+def tkMhaH100LCFFwd64() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100LCF.lean:84-107 -- D = 64, KV tiles of 192 rows, 3072 / 192 = 16 of them."""
+    return _mhaH100LcfFwd("tkMhaH100LCFFwd64", 64, 192, 16,
+                          "=== ThunderKittens mha_h100_lcf forward (D=64, KV tile 192) ===", 0.125)
+
+
+def tkMhaH100LCFFwd128() -> Kernel:
+    """Tyr/GPU/Kernels/MhaH100LCF.lean:109-132 -- D = 128, KV tiles of 128 rows, 3072 / 128 = 24 of them."""
+    return _mhaH100LcfFwd("tkMhaH100LCFFwd128", 128, 128, 24,
+                          "=== ThunderKittens mha_h100_lcf forward (D=128, KV tile 128) ===", 0.08838834764)
+
+
+def tkH100Bf16GemmFwd() -> Kernel:
+    """Tyr/GPU/Kernels/Bf16Gemm.lean:19-73 over GemmCommon.lean:22-69 -- C tile 128 x 256 from A [128, 64] and
+    B [256, 64] (B is N x K) slices over 4 K blocks, f32 accumulate, bf16 out."""
+    k = KernelBuilder("tkH100Bf16GemmFwd")
+    aPtr = k.gptr("BFloat16", "aPtr")
+    bPtr = k.gptr("BFloat16", "bPtr")
+    cPtr = k.gptr("BFloat16", "cPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    accum, coord = _tiledAccumulator(
+        k, "=== H100 BF16 GEMM ===",
+        "ThunderKittens bf16_h100 producer/consumer tile, expressed as a single CTA-local tiled mainloop",
+        aPtr, bPtr, "BFloat16", 128, 64, 256, 4)
+    # storeConvertedTile (GemmCommon.lean:58-69)
+    out = k.allocRT("BFloat16", 128, 256)
+    outShared = k.allocST("BFloat16", 128, 256)
+    k.convert(out, accum)
+    k.store(outShared, out)
+    k.storeGlobal(cPtr, outShared, coord)
+    return k.build()
+
+
 def _tiledAccumulator(k: KernelBuilder, banner, sourceNote, aPtr, bPtr, inDtype, tileM, tileK, tileN, kBlocks):
     """Tyr/GPU/Kernels/GemmCommon.lean:22-56 -- A tile [tileM, tileK], B tile [tileN, tileK] (B is N x K),
     f32 accumulator over kBlocks slices."""
@@ -552,7 +662,16 @@ CITES = {
     "tkMhaH100Fwd2Block": "Tyr/GPU/Kernels/MhaH100.lean:130-190 (runner Examples/GPU/RunMhaH100.lean:112)",
     "tkMhaH100BwdPrep2Block": "Tyr/GPU/Kernels/MhaH100.lean:192-227 (runner Examples/GPU/RunMhaH100.lean:119)",
     "tkMhaH100Bwd2BlockPartials": "Tyr/GPU/Kernels/MhaH100.lean:229-344 (runner Examples/GPU/RunMhaH100.lean:126)",
+    "tkFlashAttnFwd12Block": "Tyr/GPU/Kernels/MhaH100.lean:347-398",
+    "tkFlashAttnFwd12BlockLse": "Tyr/GPU/Kernels/MhaH100.lean:400-457 (runner Examples/GPU/RunMhaH100Seq768.lean:102)",
+    "tkMhaH100Fwd12Block": "Tyr/GPU/Kernels/MhaH100.lean:459-519 (runner Examples/GPU/RunMhaH100Seq768.lean:108)",
+    "tkMhaH100Bwd12BlockPartials": "Tyr/GPU/Kernels/MhaH100.lean:521-640 (runner Examples/GPU/RunMhaH100Seq768.lean:119)",
+    "tkMhaH100LCFFwd64": "Tyr/GPU/Kernels/MhaH100LCF.lean:84-107 (run by a group of 2 waves, K and V read from LDS by the products)",
+    "tkMhaH100LCFFwd128": "Tyr/GPU/Kernels/MhaH100LCF.lean:109-132 (run by a group of 2 waves, K and V read from LDS by the products)",
+    "tkH100Bf16GemmFwd": "Tyr/GPU/Kernels/Bf16Gemm.lean:64-73 over GemmCommon.lean:22-69 (run by a group of 4 waves, B read from LDS by the products)",
 }
 ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, gemmFp8E4M3Fwd, tkH100Fp8ScaledGemmFwd,
        tkFlashAttnFwd2Block, tkFlashAttnFwd2BlockLse,
-       tkMhaH100Fwd2Block, tkMhaH100BwdPrep2Block, tkMhaH100Bwd2BlockPartials)
+       tkMhaH100Fwd2Block, tkMhaH100BwdPrep2Block, tkMhaH100Bwd2BlockPartials,
+       tkFlashAttnFwd12Block, tkFlashAttnFwd12BlockLse, tkMhaH100Fwd12Block, tkMhaH100Bwd12BlockPartials,
+       tkMhaH100LCFFwd64, tkMhaH100LCFFwd128, tkH100Bf16GemmFwd)
