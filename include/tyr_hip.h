@@ -340,6 +340,23 @@ int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c,
                      uint64_t M, uint64_t N, uint64_t K,
                      float scale_a, float scale_b, int trans_b, void* stream);
 
+/* The other epilogues of the reference's fp8 GEMM family on the same mainloop:
+ *     C[m, n] = out_dtype( scale * row_scale[m] * col_scale[n] * sum_k Aq[m, k] Bq[k, n] )
+ *   - `tkH100Fp8E4M3GemmFwd` (Tyr/GPU/Kernels/PrecisionGemm.lean:78-89): E4M3 output, no scales
+ *     (out_dtype = TYR_HIP_OUT_E4M3; round to nearest even, saturating at +-448);
+ *   - `tkH100Fp8ScaledGemmFwd` (Tyr/GPU/Kernels/PrecisionGemm.lean:97-115 with the epilogue of
+ *     Tyr/GPU/Kernels/GemmCommon.lean:83-133): per-row and per-column f32 dequantisation scales, f32 output
+ *     (out_dtype = TYR_HIP_OUT_F32, row_scale [M], col_scale [N]);
+ *   - tyr_hip_gemm_fp8 is this call with scale = scale_a * scale_b, no vectors, TYR_HIP_OUT_BF16.
+ * row_scale / col_scale: device f32 vectors or NULL (= all ones); col_scale 16-byte aligned.
+ * c: [M, N] of the output type.  Shapes as tyr_hip_gemm_fp8.
+ */
+enum tyr_hip_out_dtype { TYR_HIP_OUT_BF16 = 0, TYR_HIP_OUT_F32 = 1, TYR_HIP_OUT_E4M3 = 2 };
+int tyr_hip_gemm_fp8_ex(const void* aq, const void* bq, void* c,
+                        uint64_t M, uint64_t N, uint64_t K,
+                        float scale, const float* row_scale, const float* col_scale, int out_dtype,
+                        int trans_b, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Calibration: the MFMA rate this device sustains on the caller's operand bits.
  *

@@ -54,6 +54,8 @@ def test_host_validation_needs_no_gpu():
     assert L.tyr_hip_gemm_force_general(prev) == 1 and L.tyr_hip_gemm_force_general(prev) == prev
     assert L.tyr_hip_gemm_fp8(p, p, None, 16, 16, 16, 1.0, 1.0, 0, None) == NULL
     assert L.tyr_hip_gemm_fp8(p, p, p, 16, 8, 16, 1.0, 1.0, 0, None) == UNSUP
+    assert L.tyr_hip_gemm_fp8_ex(p, p, p, 16, 16, 16, 1.0, None, None, 7, 0, None) == UNSUP           # unknown output type
+    assert L.tyr_hip_gemm_fp8_ex(p, p, p, 16, 16, 16, 1.0, None, p + 4, 1, 0, None) == MISAL          # column scales: 16-byte rows
     assert L.tyr_hip_flash_attn_fwd(p, p, None, p, None, 1, 1, 16, 128, 1, 0.1, None) == NULL
     assert L.tyr_hip_flash_attn_fwd(p, p, p, p, None, 1, 1, 0, 128, 1, 0.1, None) == SHAPE
     assert L.tyr_hip_flash_attn_fwd(p, p, p, p, None, 1, 1, 16, 96, 1, 0.1, None) == UNSUP

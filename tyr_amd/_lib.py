@@ -14,7 +14,7 @@ SYMBOLS = (
     "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_fwd_gqa", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
     "tyr_hip_flash_attn_bwd_gqa", "tyr_hip_flash_attn_fwd_mask", "tyr_hip_flash_attn_bwd_mask",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
-    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_bf16_batched", "tyr_hip_gemm_force_general", "tyr_hip_gemm_fp8",
+    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_bf16_batched", "tyr_hip_gemm_force_general", "tyr_hip_gemm_fp8", "tyr_hip_gemm_fp8_ex",
     "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy", "tyr_hip_mfma_sustain",
 )
 
@@ -73,6 +73,8 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_gemm_force_general.restype = ci
     L.tyr_hip_gemm_fp8.argtypes = [vp, vp, vp, u64, u64, u64, f32, f32, ci, vp]
     L.tyr_hip_gemm_fp8.restype = ci
+    L.tyr_hip_gemm_fp8_ex.argtypes = [vp, vp, vp, u64, u64, u64, f32, vp, vp, ci, ci, vp]
+    L.tyr_hip_gemm_fp8_ex.restype = ci
     L.tyr_hip_decode_rope_append.argtypes = [vp] * 8 + [u64] * 6 + [vp]
     L.tyr_hip_decode_rope_append.restype = ci
     L.tyr_hip_rope_fwd.argtypes = [vp, vp, vp, vp, u64, u64, u64, u64, ci, vp]

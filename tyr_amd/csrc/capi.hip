@@ -394,14 +394,24 @@ int tyr_hip_gemm_force_general(int on) { return tyr::set_gemm_general_only(on); 
 
 int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c, uint64_t M, uint64_t N, uint64_t K,
                      float scale_a, float scale_b, int trans_b, void* stream) {
+    return tyr_hip_gemm_fp8_ex(aq, bq, c, M, N, K, scale_a * scale_b, nullptr, nullptr, TYR_HIP_OUT_BF16, trans_b, stream);
+}
+
+int tyr_hip_gemm_fp8_ex(const void* aq, const void* bq, void* c, uint64_t M, uint64_t N, uint64_t K,
+                        float scale, const float* row_scale, const float* col_scale, int out_dtype,
+                        int trans_b, void* stream) {
     if (!aq || !bq || !c) return TYR_HIP_ERR_NULL_POINTER;
     if (M == 0 || N == 0 || K == 0) return TYR_HIP_ERR_BAD_SHAPE;
     if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return TYR_HIP_ERR_BAD_SHAPE;
     if (((M + 255) / 256) * ((N + 255) / 256) > (uint64_t)INT_MAX) return TYR_HIP_ERR_BAD_SHAPE;
     if (K % 16 != 0 || N % 16 != 0) return TYR_HIP_ERR_UNSUPPORTED;
+    if (out_dtype != TYR_HIP_OUT_BF16 && out_dtype != TYR_HIP_OUT_F32 && out_dtype != TYR_HIP_OUT_E4M3)
+        return TYR_HIP_ERR_UNSUPPORTED;
     if (!aligned16(aq) || !aligned16(bq) || !aligned16(c)) return TYR_HIP_ERR_MISALIGNED;
-    const int rc = tyr::launch_gemm_fp8(aq, bq, c, (int)M, (int)N, (int)K, scale_a * scale_b,
-                                        trans_b != 0, static_cast<hipStream_t>(stream));
+    if ((row_scale && (reinterpret_cast<uintptr_t>(row_scale) & 3u)) || (col_scale && !aligned16(col_scale)))
+        return TYR_HIP_ERR_MISALIGNED;
+    const int rc = tyr::launch_gemm_fp8(aq, bq, c, (int)M, (int)N, (int)K, scale, trans_b != 0, row_scale, col_scale,
+                                        out_dtype, static_cast<hipStream_t>(stream));
     return rc == 0 ? TYR_HIP_OK : TYR_HIP_ERR_LAUNCH;
 }
 

@@ -223,6 +223,56 @@ __device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], f
     }
 }
 
+// Epilogue variants of the fp8 GEMM beyond "one scalar, bf16 out": per-row and per-column scales and the
+// output element type.  The common case (no vectors, bf16) takes store_quadrant_bf16 above.
+struct GemmEpilogue {
+    float scale;                 // multiplies every element
+    const float* row_scale;      // [M] or nullptr
+    const float* col_scale;      // [N] or nullptr
+    int out;                     // 0 = bf16, 1 = f32, 2 = e4m3 (round to nearest even, saturating at +-448)
+    __device__ __host__ bool plain_bf16() const { return out == 0 && row_scale == nullptr && col_scale == nullptr; }
+};
+// One wave's 128x128 accumulator quadrant (layout as in store_quadrant_bf16) written straight from registers:
+// a lane stores the 4 consecutive n of a register group of its row.  gm0 / gn0 = global row / column of the
+// quadrant's first element; M, N = extents of C (row pitch N elements).
+__device__ __forceinline__ void store_quadrant_ex(const f32x16 (&acc)[4][4], const GemmEpilogue& ep, void* C, int M, int N,
+                                                  int gm0, int gn0, int lane) {
+    const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int gm = gm0 + i * 32 + r;
+        if (gm >= M) continue;
+        const float rs = ep.scale * (ep.row_scale ? ep.row_scale[gm] : 1.0f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int gn = gn0 + j * 32 + q4 * 8 + g * 4;
+                if (gn >= N) continue;                       // N is a multiple of 16: a group of 4 is inside or outside
+                float v[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) v[x] = acc[i][j][q4 * 4 + x] * rs;
+                if (ep.col_scale) {
+                    const f32x4 cs = *reinterpret_cast<const f32x4*>(ep.col_scale + gn);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) v[x] *= cs[x];
+                }
+                const size_t at = (size_t)gm * N + gn;
+                if (ep.out == 1) {
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(C) + at) = f32x4{v[0], v[1], v[2], v[3]};
+                } else if (ep.out == 2) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) v[x] = v[x] != v[x] ? v[x] : fminf(fmaxf(v[x], -448.0f), 448.0f);
+                    int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+                    w = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true);
+                    *reinterpret_cast<int*>(static_cast<uint8_t*>(C) + at) = w;
+                } else {
+                    st_global_8(static_cast<uint16_t*>(C) + at, u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])});
+                }
+            }
+    }
+}
+
 // Grid remap for the 8 XCDs of an MI355X: consecutive workgroup ids are dealt round-robin
 // to the XCDs, each with its own L2.  This returns a logical id such that the workgroups
 // that land on one XCD cover one contiguous range of logical ids (so neighbours in the

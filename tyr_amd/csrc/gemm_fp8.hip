@@ -41,7 +41,8 @@ __device__ __forceinline__ void transpose4x4_b8(uint32_t x0, uint32_t x1, uint32
 template <bool TRANS_B, bool EDGE>
 __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, int tiles_m, int tiles_n, float scale) {
+    int M, int N, int K, int tiles_m, int tiles_n, GemmEpilogue ep) {
+    const float scale = ep.scale;
     using namespace gemm8;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -177,6 +178,10 @@ __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
         __syncthreads();
     }
 
+    if (!ep.plain_bf16()) {
+        store_quadrant_ex(acc, ep, C, M, N, m0 + wm * 128, n0 + wn * 128, lane);
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int gm = m0 + wm * 128 + i * 32 + r;
@@ -213,7 +218,8 @@ constexpr int GROUP_M = 4;
 template <bool TRANS_B, bool K_TAIL>
 __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, int tiles_m, int tiles_n, float scale) {
+    int M, int N, int K, int tiles_m, int tiles_n, GemmEpilogue ep) {
+    const float scale = ep.scale;
     using namespace gemm8f;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -384,13 +390,18 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     }
 #undef TYR_FENCE
 
+    if (!ep.plain_bf16()) {
+        store_quadrant_ex(acc, ep, C, M, N, m0 + wm * 128, n0 + wn * 128, lane);
+        return;
+    }
     store_quadrant_bf16(acc, scale, lds + w * kEpilogueScratchBytes,
                         C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
                         M - (m0 + wm * 128), N - (n0 + wn * 128));
 }
 
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
-                    int trans_b, hipStream_t stream) {
+                    int trans_b, const float* row_scale, const float* col_scale, int out_kind, hipStream_t stream) {
+    const GemmEpilogue ep{scale, row_scale, col_scale, out_kind};
     using namespace gemm8;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const bool edge = (M % BM) || (N % BN) || (K % BK);
@@ -414,7 +425,7 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm8f::LDS_BYTES);                   \
             if (attr != hipSuccess) return -1;                                                    \
             hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB, KT>), grid, block, gemm8f::LDS_BYTES, stream, \
-                               A, Bp, Cp, M, N, K, tiles_m, tiles_n, scale);                      \
+                               A, Bp, Cp, M, N, K, tiles_m, tiles_n, ep);                         \
         } while (0)
         const bool k_tail = K % gemm8f::BK != 0;
         if (trans_b) { if (k_tail) TYR_GEMM8_FAST(true, true); else TYR_GEMM8_FAST(true, false); }
@@ -429,7 +440,7 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);                               \
         if (attr != hipSuccess) return -1;                                                        \
         hipLaunchKernelGGL((gemm_fp8_kernel<TB, ED>), grid, block, LDS_BYTES, stream, A, Bp, Cp,  \
-                           M, N, K, tiles_m, tiles_n, scale);                                     \
+                           M, N, K, tiles_m, tiles_n, ep);                                        \
     } while (0)
     if (trans_b) { if (edge) TYR_GEMM8_LAUNCH(true, true); else TYR_GEMM8_LAUNCH(true, false); }
     else         { if (edge) TYR_GEMM8_LAUNCH(false, true); else TYR_GEMM8_LAUNCH(false, false); }

@@ -365,6 +365,39 @@ def gemm_fp8(aq, bq, scale_a: float, scale_b: float, trans_b: bool = False, stre
     return c
 
 
+@_on_launch_stream
+def gemm_fp8_scaled(aq, bq, row_scale=None, col_scale=None, scale: float = 1.0, out_dtype=torch.float32,
+                    trans_b: bool = False, stream=None):
+    """C = gemmFp8Scaled aq bq rowScale colScale: out_dtype(scale * rowScale[m] * colScale[n] * (aq bq)[m, n]).
+
+    The per-row / per-column dequantisation epilogue of `tkH100Fp8ScaledGemmFwd` (f32 out) and, with no scales and
+    out_dtype = torch.float8_e4m3fn, the E4M3 epilogue of `tkH100Fp8E4M3GemmFwd`.  aq e4m3 [M,K]; bq e4m3 [K,N] (or
+    [N,K] with trans_b); row_scale f32 [M], col_scale f32 [N] or None."""
+    _check(aq, "a", torch.float8_e4m3fn, 2)
+    _check(bq, "b", torch.float8_e4m3fn, 2)
+    M, K = aq.shape
+    N, Kb = (bq.shape[0], bq.shape[1]) if trans_b else (bq.shape[1], bq.shape[0])
+    if Kb != K:
+        raise TyrGpuError("a and b have mismatched inner dimensions")
+    kinds = {torch.bfloat16: 0, torch.float32: 1, torch.float8_e4m3fn: 2}
+    if out_dtype not in kinds:
+        raise TyrGpuError("out_dtype must be bfloat16, float32 or float8_e4m3fn")
+    ptrs = []
+    for t, n, ln in ((row_scale, "rowScale", M), (col_scale, "colScale", N)):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _check(t, n, torch.float32, 1)
+        if t.numel() != ln:
+            raise TyrGpuError(f"{n} must hold one scale per {'row' if ln == M else 'column'}")
+        ptrs.append(t.data_ptr())
+    c = torch.empty((M, N), dtype=out_dtype, device=aq.device)
+    rc = _lib.load().tyr_hip_gemm_fp8_ex(aq.data_ptr(), bq.data_ptr(), c.data_ptr(), M, N, K, float(scale), ptrs[0], ptrs[1],
+                                         kinds[out_dtype], int(bool(trans_b)), _stream(stream))
+    _raise(rc, "gemmFp8Scaled")
+    return c
+
+
 def quantize_e4m3(x: torch.Tensor):
     """Per-tensor absmax quantisation used by the harness: s = absmax/448, xq = e4m3fn(x / s)."""
     s = float(x.abs().max()) / 448.0
