@@ -528,5 +528,64 @@ lean_object* lean_tyr_gpu_gemm_fp8(uint64_t M, uint64_t N, uint64_t K, b_lean_ob
     }
 }
 
+// matmulBf16 {Bt M N K} a b stream : IO (T #[Bt,M,N])   -- `lean_torch_matmul` on rank-3 operands, one launch
+lean_object* lean_tyr_gpu_matmul_bf16(uint64_t Bt, uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a,
+                                      b_lean_obj_arg b, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b);
+        std::string err;
+        if (!check(a_, "a", torch::kBFloat16, err) || !check(b_, "b", torch::kBFloat16, err))
+            return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
+        auto c = torch::empty({(int64_t)Bt, (int64_t)M, (int64_t)N}, a_.options());
+        const int rc = tyr_hip_gemm_bf16_batched(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), Bt, M, N, K, M * K, K * N,
+                                                 M * N, 0, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("matmulBf16", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gemmFp8Scaled {M N K} a b rowScale colScale stream : IO (T #[M,N])   -- f32 out, per-row x per-column scales
+lean_object* lean_tyr_gpu_gemm_fp8_scaled(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a, b_lean_obj_arg b,
+                                          b_lean_obj_arg row_scale, b_lean_obj_arg col_scale, uint64_t stream,
+                                          lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b), r_ = borrowTensor(row_scale), c_ = borrowTensor(col_scale);
+        std::string err;
+        if (!check(a_, "a", torch::kFloat8_e4m3fn, err) || !check(b_, "b", torch::kFloat8_e4m3fn, err) ||
+            !check(r_, "rowScale", torch::kFloat32, err) || !check(c_, "colScale", torch::kFloat32, err))
+            return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
+        auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options().dtype(torch::kFloat32));
+        const int rc = tyr_hip_gemm_fp8_ex(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, 1.0f, r_.data_ptr<float>(),
+                                           c_.data_ptr<float>(), TYR_HIP_OUT_F32, 0, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gemmFp8Scaled", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// gemmFp8E4M3 {M N K} a b scale stream : IO (T #[M,N])   -- E4M3 out (tkH100Fp8E4M3GemmFwd)
+lean_object* lean_tyr_gpu_gemm_fp8_e4m3(uint64_t M, uint64_t N, uint64_t K, b_lean_obj_arg a, b_lean_obj_arg b,
+                                        double scale, uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto a_ = borrowTensor(a), b_ = borrowTensor(b);
+        std::string err;
+        if (!check(a_, "a", torch::kFloat8_e4m3fn, err) || !check(b_, "b", torch::kFloat8_e4m3fn, err))
+            return io_error(err);
+        LaunchStreamScope on_stream(stream, a_);   // outputs and scratch belong to the launch stream
+        auto c = torch::empty({(int64_t)M, (int64_t)N}, a_.options());
+        const int rc = tyr_hip_gemm_fp8_ex(a_.data_ptr(), b_.data_ptr(), c.data_ptr(), M, N, K, (float)scale, nullptr,
+                                           nullptr, TYR_HIP_OUT_E4M3, 0, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("gemmFp8E4M3", rc);
+        return lean_io_result_mk_ok(giveTensor(std::move(c)));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 }  // extern "C"
 #endif  // TYR_HAVE_LEAN

@@ -170,4 +170,23 @@ opaque gemmBf16NT {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[N, K]) (stream
 opaque gemmFp8 {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (scaleA scaleB : Float)
     (stream : CudaStream) : IO (T #[M, N])
 
+/-- Batched matmul of rank-3 operands in one launch: `C[i] = A[i] · B[i]`. GPU twin of `torch.matmul`
+    (`lean_torch_matmul`, `cc/src/tyr.cpp:1565-1570`) for `[Bt, M, K] × [Bt, K, N]`. -/
+@[extern "lean_tyr_gpu_matmul_bf16"]
+opaque matmulBf16 {Bt M N K : UInt64} (a : @& T #[Bt, M, K]) (b : @& T #[Bt, K, N]) (stream : CudaStream)
+    : IO (T #[Bt, M, N])
+
+/-- FP8 GEMM with per-row and per-column f32 dequantisation scales and f32 output:
+    `C[m,n] = rowScale[m] · colScale[n] · (Aq · Bq)[m,n]`, the epilogue of `tkH100Fp8ScaledGemmFwd`
+    (`Tyr/GPU/Kernels/PrecisionGemm.lean:97-115`, `GemmCommon.lean:83-133`). -/
+@[extern "lean_tyr_gpu_gemm_fp8_scaled"]
+opaque gemmFp8Scaled {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (rowScale : @& T #[M])
+    (colScale : @& T #[N]) (stream : CudaStream) : IO (T #[M, N])
+
+/-- FP8 GEMM with E4M3 output (round to nearest even, saturating at ±448): `tkH100Fp8E4M3GemmFwd`
+    (`Tyr/GPU/Kernels/PrecisionGemm.lean:78-89`). `scale` multiplies the f32 accumulators before the cast. -/
+@[extern "lean_tyr_gpu_gemm_fp8_e4m3"]
+opaque gemmFp8E4M3 {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (scale : Float)
+    (stream : CudaStream) : IO (T #[M, N])
+
 end Tyr.GPU.GFX950
