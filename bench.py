@@ -54,7 +54,10 @@ TRAFFIC = {"attn_fwd_causal": 1_073_162_240 + 272_629_760, "gqa_decode": 1_090_8
            "rope_kernel<bf16>": 270_592_000 + 268_437_504,
            "layernorm_residual_kernel<2>": 268_521_472 + 268_435_456,
            "copy_kernel": 1_073_784_832 + 1_073_848_320,
-           "decode_rope_append_kernel + gqa_decode_split_kernel<8>": 423_680 + 393_216 + 1_090_152_448 + 270_336}
+           "decode_rope_append_kernel + gqa_decode_split_kernel<8>": 423_680 + 393_216 + 1_090_152_448 + 270_336,
+           "gqa_decode_split4": 1_085_655_040 + 2_228_224 + 2_403_328 + 294_912,       # split pass + combine pass
+           "gqa_decode_small_batch": 542_947_328 + 589_824 + 601_088 + 36_864,
+           "dsl_simple_gemm": 77_063_987 + 268_435_456}
 
 
 def _events(torch, n):
@@ -301,7 +304,9 @@ def _wl_decode(torch, tyr, steps, warmup, cpu, parity, splits, shape=(32, 32, 8,
                             "combine pass merges them with the LSE algebra; both passes are inside the timed step")},
         "roofline": {"bound": "hbm", "kernel": "gqa_decode_split_kernel<8>" + ("" if used == 1 else " + gqa_decode_combine_kernel"),
                      "achieved": gbs, "peak": PEAK["hbm"], "unit": "GB/s", "frac": gbs / PEAK["hbm"],
-                     "traffic": TRAFFIC["gqa_decode"] if (used == 1 and shape == (32, 32, 8, 8192, 128)) else None},
+                     "traffic": {((32, 32, 8, 8192, 128), 1): TRAFFIC["gqa_decode"],
+                                 ((32, 32, 8, 8192, 128), 4): TRAFFIC["gqa_decode_split4"],
+                                 ((4, 32, 8, 32768, 128), 8): TRAFFIC["gqa_decode_small_batch"]}.get((shape, used))},
     }
     if parity:
         import numpy as np
