@@ -455,6 +455,20 @@ def _train_setup(torch, tyr, shape, causal, noise):
     return sc, target, init
 
 
+def _train_step_fused(torch, tyr, masters, lows, target, lr, causal, sc):
+    """The same step with the element-wise chains as this library's two fused kernels: the bf16 copies of the masters come
+    out of the SGD kernel of the previous step, loss and dO out of one pass over O and the target."""
+    o, lse = tyr.flash_attn_fwd(lows[0], lows[1], lows[2], causal=causal, scale=sc)
+    loss, d_o = tyr.mse_loss_grad(o, target)
+    grads = tyr.flash_attn_bwd(lows[0], lows[1], lows[2], o, lse, d_o, causal=causal, scale=sc)
+    new_m, new_l = [], []
+    for m, g in zip(masters, grads):
+        a, b = tyr.sgd_step(m, g, lr, in_place=True)
+        new_m.append(a)
+        new_l.append(b)
+    return new_m, new_l, loss
+
+
 def _train_step(torch, tyr, qM, kM, vM, target, lr, causal, sc):
     """oneKernelTrainStep (Examples/GPU/RunMhaH100Train.lean:77-93): cast the f32 masters to bf16, forward, loss =
     0.5 mean((O - target)^2), dO = (O - target) / numel in bf16, backward, SGD on the masters.  The casts, the loss and the
@@ -474,9 +488,16 @@ def _wl_train(torch, tyr, steps, warmup, cpu, parity, shape, causal, lr, label):
     state = [t.clone() for t in init]
     losses = []
 
-    def fn():
+    def fn_torch_elementwise():
         q, k, v, loss = _train_step(torch, tyr, state[0], state[1], state[2], target, lr, causal, sc)
         state[0], state[1], state[2] = q, k, v
+        losses.append(loss)
+    _, ms_torch_elementwise = time_steps(torch, fn_torch_elementwise, max(5, steps // 3), 2)
+    fstate = {"m": [t.clone() for t in init]}
+    fstate["l"] = [t.to(torch.bfloat16) for t in fstate["m"]]
+
+    def fn():
+        fstate["m"], fstate["l"], loss = _train_step_fused(torch, tyr, fstate["m"], fstate["l"], target, lr, causal, sc)
         losses.append(loss)
     wall, ms = time_steps(torch, fn, steps, warmup)
     flop = 14.0 * B * H * N * N * D / (2.0 if causal else 1.0)
@@ -485,10 +506,12 @@ def _wl_train(torch, tyr, steps, warmup, cpu, parity, shape, causal, lr, label):
         "metric": "train step TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
         "dtype": "bf16 kernels, f32 master weights",
         "config": {"workload": f"attention train step ({label}): cast + forward + MSE loss + backward + SGD, "
-                               f"B={B} H={H} N={N} D={D}, {'causal' if causal else 'non-causal'}",
+                               f"B={B} H={H} N={N} D={D}, {'causal' if causal else 'non-causal'}; element-wise chains fused "
+                               f"(tyr_hip_mse_loss_grad, tyr_hip_sgd_step)",
+                   "ms_per_step_with_libtorch_elementwise": ms_torch_elementwise,
                    "flop_convention": "forward 4 + backward 10 = 14*B*H*N^2*D" + ("/2 (causal half)" if causal else ""),
                    "kernel_ms_per_step": ms, "kernel_steps_per_sec": 1e3 / ms, "lr": lr},
-        "roofline": _mfma_roofline(torch, "mfma_bf16", "flash_attn_fwd_kernel + " + BWD_KERNELS + " + LibTorch elementwise",
+        "roofline": _mfma_roofline(torch, "mfma_bf16", "flash_attn_fwd_kernel + " + BWD_KERNELS + " + mse_grad_kernel + sgd_kernel",
                                    tf, None),
     }
     if parity:
@@ -497,9 +520,15 @@ def _wl_train(torch, tyr, steps, warmup, cpu, parity, shape, causal, lr, label):
         import numpy as np
         import oracle
         st = [t.clone() for t in init]
-        ls = []
+        fm = [t.clone() for t in init]
+        fl = [t.to(torch.bfloat16) for t in fm]
+        ls, same = [], True
         for _ in range(12):
             st[0], st[1], st[2], loss = _train_step(torch, tyr, st[0], st[1], st[2], target, lr, causal, sc)
+            fm, fl, floss = _train_step_fused(torch, tyr, fm, fl, target, lr, causal, sc)
+            # the fused element-wise kernels reproduce the LibTorch chain bit for bit, so both runs stay identical
+            same = same and all(bool(torch.equal(a, b)) for a, b in zip(st, fm)) and \
+                abs(float(loss) - float(floss)) <= 1e-5 * abs(float(loss))
             ls.append(float(loss))
         b, h = B - 1, H - 1
         qb, kb, vb = (t.to(torch.bfloat16) for t in init)
@@ -511,8 +540,10 @@ def _wl_train(torch, tyr, steps, warmup, cpu, parity, shape, causal, lr, label):
         got = tyr.flash_attn_bwd(qb, kb, vb, o, lse, d_o, causal=causal, scale=sc)
         rel = max(float(np.linalg.norm(g_[b, h].cpu().float().numpy() - w_[0, 0]) / max(np.linalg.norm(w_[0, 0]), 1e-30))
                   for g_, w_ in zip(got, want))
-        res["parity"] = _parity(tol=1e-2, rel_fro=rel, ok=rel <= 1e-2 and ls[-1] < ls[0], init_loss=ls[0], final_loss=ls[-1],
-                                sample=f"12 steps from the initial state (loss must fall, as the reference's runner demands); "
+        res["parity"] = _parity(tol=1e-2, rel_fro=rel, ok=rel <= 1e-2 and ls[-1] < ls[0] and same, init_loss=ls[0], final_loss=ls[-1],
+                                fused_equals_libtorch_chain=float(same),
+                                sample=f"12 steps from the initial state, once with LibTorch element-wise calls and once with the fused "
+                                       f"kernels (masters must stay bit-identical; loss must fall, as the reference's runner demands); "
                                        f"dQ, dK, dV of the first step, head ({b},{h}), against oracle.attn_bwd_f64")
     if cpu:
         from oracle import libtorch_path as lt

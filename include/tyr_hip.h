@@ -358,6 +358,27 @@ int tyr_hip_gemm_fp8_ex(const void* aq, const void* bq, void* c,
                         int trans_b, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * The element-wise half of the attention train step, fused.
+ *
+ * The reference's `oneKernelTrainStep` (Examples/GPU/RunMhaH100Train.lean:77-93) surrounds its forward
+ * and backward kernels with LibTorch element-wise calls; these two entry points are those chains as one
+ * streaming pass each, with bit-identical results for dO and the parameters.
+ *
+ * tyr_hip_mse_loss_grad -- `lossAndGradOut` (:60-67):
+ *     diff = f32(out) - f32(target);  *loss = 0.5 * mean(diff^2);  d_out = bf16(diff / n)
+ *   out, target, d_out : bf16 [n] (any shape, n elements, n % 8 == 0);  loss : device f32 scalar
+ *   workspace : tyr_hip_mse_loss_grad_workspace_bytes(n) bytes of device scratch (per-workgroup partial sums)
+ * tyr_hip_sgd_step -- `sgdUpdate` (:69-70) plus the bf16 cast of the next step (:83-85):
+ *     param_out = param - (f32(grad) * lr);  param_out_bf16 = bf16(param_out)  (skipped when NULL)
+ *   param, param_out : f32 [n] (param_out may alias param);  grad, param_out_bf16 : bf16 [n];  n % 8 == 0
+ */
+size_t tyr_hip_mse_loss_grad_workspace_bytes(uint64_t n);
+int tyr_hip_mse_loss_grad(const void* out, const void* target, void* d_out, float* loss, uint64_t n,
+                          void* workspace, size_t workspace_bytes, void* stream);
+int tyr_hip_sgd_step(const float* param, const void* grad, float lr, float* param_out, void* param_out_bf16,
+                     uint64_t n, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Calibration: the MFMA rate this device sustains on the caller's operand bits.
  *
  * No counterpart in the reference; it belongs to the measurement side, where the reference's

@@ -51,6 +51,19 @@ def sdpa_4d_backward(q, k, v, d_o, is_causal: bool):
     return q32.grad, k32.grad, v32.grad
 
 
+def loss_and_grad_out(out, target):
+    """`lossAndGradOut` (Examples/GPU/RunMhaH100Train.lean:60-67), call for call: (loss, dO bf16)."""
+    out32, tgt32 = out.float(), target.float()
+    diff = out32 - tgt32
+    loss = (diff * diff).mean() * 0.5
+    return loss, (diff / float(diff.numel())).to(torch.bfloat16)
+
+
+def sgd_update(param, grad, lr: float):
+    """`sgdUpdate` (Examples/GPU/RunMhaH100Train.lean:69-70) on an f32 master and a bf16 gradient."""
+    return param - (grad.float() * lr)
+
+
 def train_step(q_m, k_m, v_m, target32, lr: float, is_causal: bool = False):
     """`oneTorchTrainStep` (Examples/GPU/RunMhaH100Train.lean:95-113): f32 SDPA of the detached masters, loss =
     0.5 mean((out - target)^2), autograd, SGD.  Returns the updated masters and the loss."""

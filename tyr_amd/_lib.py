@@ -15,7 +15,7 @@ SYMBOLS = (
     "tyr_hip_flash_attn_bwd_gqa", "tyr_hip_flash_attn_fwd_mask", "tyr_hip_flash_attn_bwd_mask",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
     "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_bf16_batched", "tyr_hip_gemm_force_general", "tyr_hip_gemm_fp8", "tyr_hip_gemm_fp8_ex",
-    "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy", "tyr_hip_mfma_sustain",
+    "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy", "tyr_hip_mfma_sustain", "tyr_hip_mse_loss_grad_workspace_bytes", "tyr_hip_mse_loss_grad", "tyr_hip_sgd_step",
 )
 
 _lib = None
@@ -85,5 +85,11 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_copy.restype = ci
     L.tyr_hip_mfma_sustain.argtypes = [vp, sz, ci, u64, u64, vp, ctypes.POINTER(ctypes.c_double), vp]
     L.tyr_hip_mfma_sustain.restype = ci
+    L.tyr_hip_mse_loss_grad_workspace_bytes.argtypes = [u64]
+    L.tyr_hip_mse_loss_grad_workspace_bytes.restype = sz
+    L.tyr_hip_mse_loss_grad.argtypes = [vp, vp, vp, vp, u64, vp, sz, vp]
+    L.tyr_hip_mse_loss_grad.restype = ci
+    L.tyr_hip_sgd_step.argtypes = [vp, vp, f32, vp, vp, u64, vp]
+    L.tyr_hip_sgd_step.restype = ci
     _lib = L
     return L

@@ -587,5 +587,47 @@ lean_object* lean_tyr_gpu_gemm_fp8_e4m3(uint64_t M, uint64_t N, uint64_t K, b_le
     }
 }
 
+// lossAndGradOut {s} out target stream : IO (T #[] x T s)   -- loss = 0.5 mean((out - target)^2), dO = bf16((out - target) / n)
+lean_object* lean_tyr_gpu_mse_loss_grad(lean_obj_arg /*shape*/, b_lean_obj_arg out, b_lean_obj_arg target, uint64_t stream,
+                                        lean_object* /*world*/) {
+    try {
+        auto o_ = borrowTensor(out), t_ = borrowTensor(target);
+        std::string err;
+        if (!check(o_, "out", torch::kBFloat16, err) || !check(t_, "target", torch::kBFloat16, err)) return io_error(err);
+        if (o_.numel() != t_.numel()) return io_error("out and target must have the same shape");
+        LaunchStreamScope on_stream(stream, o_);   // outputs and scratch belong to the launch stream
+        auto d_o = torch::empty_like(o_);
+        auto loss = torch::empty({}, o_.options().dtype(torch::kFloat32));
+        const size_t ws_bytes = tyr_hip_mse_loss_grad_workspace_bytes((uint64_t)o_.numel());
+        auto ws = torch::empty({(int64_t)(ws_bytes ? ws_bytes : 16)}, o_.options().dtype(torch::kUInt8));
+        const int rc = tyr_hip_mse_loss_grad(o_.data_ptr(), t_.data_ptr(), d_o.data_ptr(), loss.data_ptr<float>(),
+                                             (uint64_t)o_.numel(), ws.data_ptr(), ws_bytes, reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("lossAndGradOut", rc);
+        return pair_result(std::move(loss), std::move(d_o));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
+// sgdUpdate {s} param grad lr stream : IO (T s x T s)   -- (param - f32(grad) * lr, its bf16 copy)
+lean_object* lean_tyr_gpu_sgd_step(lean_obj_arg /*shape*/, b_lean_obj_arg param, b_lean_obj_arg grad, double lr,
+                                   uint64_t stream, lean_object* /*world*/) {
+    try {
+        auto p_ = borrowTensor(param), g_ = borrowTensor(grad);
+        std::string err;
+        if (!check(p_, "param", torch::kFloat32, err) || !check(g_, "grad", torch::kBFloat16, err)) return io_error(err);
+        if (p_.numel() != g_.numel()) return io_error("param and grad must have the same shape");
+        LaunchStreamScope on_stream(stream, p_);   // outputs and scratch belong to the launch stream
+        auto p_new = torch::empty_like(p_);
+        auto p_low = torch::empty_like(g_);
+        const int rc = tyr_hip_sgd_step(p_.data_ptr<float>(), g_.data_ptr(), (float)lr, p_new.data_ptr<float>(), p_low.data_ptr(),
+                                        (uint64_t)p_.numel(), reinterpret_cast<void*>(stream));
+        if (rc != TYR_HIP_OK) return status_error("sgdUpdate", rc);
+        return pair_result(std::move(p_new), std::move(p_low));
+    } catch (const std::exception& e) {
+        return io_error(e.what());
+    }
+}
+
 }  // extern "C"
 #endif  // TYR_HAVE_LEAN

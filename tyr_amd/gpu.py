@@ -398,6 +398,42 @@ def gemm_fp8_scaled(aq, bq, row_scale=None, col_scale=None, scale: float = 1.0, 
     return c
 
 
+@_on_launch_stream
+def mse_loss_grad(out, target, stream=None):
+    """(loss, dO) = lossAndGradOut out target: loss = 0.5 mean((out - target)^2) as an f32 scalar tensor,
+    dO = bf16((out - target) / numel).  out, target bf16, same shape, numel % 8 == 0."""
+    _check(out, "out", torch.bfloat16)
+    _check(target, "target", torch.bfloat16)
+    if out.shape != target.shape:
+        raise TyrGpuError("out and target must have the same shape")
+    lib = _lib.load()
+    n = out.numel()
+    d_out = torch.empty_like(out)
+    loss = torch.empty((), dtype=torch.float32, device=out.device)
+    ws = torch.empty((max(int(lib.tyr_hip_mse_loss_grad_workspace_bytes(n)), 16),), dtype=torch.uint8, device=out.device)
+    rc = lib.tyr_hip_mse_loss_grad(out.data_ptr(), target.data_ptr(), d_out.data_ptr(), loss.data_ptr(), n, ws.data_ptr(),
+                                   ws.numel(), _stream(stream))
+    _raise(rc, "lossAndGradOut")
+    return loss, d_out
+
+
+@_on_launch_stream
+def sgd_step(param, grad, lr: float, in_place: bool = False, stream=None):
+    """(param', bf16 param') = sgdUpdate param grad lr: param' = param - f32(grad) * lr for an f32 master and a bf16
+    gradient of the same shape, together with the bf16 cast the next step's kernels take.  ``in_place`` overwrites
+    ``param`` instead of allocating."""
+    _check(param, "param", torch.float32)
+    _check(grad, "grad", torch.bfloat16)
+    if param.shape != grad.shape:
+        raise TyrGpuError("param and grad must have the same shape")
+    out = param if in_place else torch.empty_like(param)
+    out_bf16 = torch.empty_like(grad)
+    rc = _lib.load().tyr_hip_sgd_step(param.data_ptr(), grad.data_ptr(), float(lr), out.data_ptr(), out_bf16.data_ptr(),
+                                      param.numel(), _stream(stream))
+    _raise(rc, "sgdUpdate")
+    return out, out_bf16
+
+
 def quantize_e4m3(x: torch.Tensor):
     """Per-tensor absmax quantisation used by the harness: s = absmax/448, xq = e4m3fn(x / s)."""
     s = float(x.abs().max()) / 448.0

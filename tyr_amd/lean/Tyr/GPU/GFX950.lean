@@ -189,4 +189,14 @@ opaque gemmFp8Scaled {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (row
 opaque gemmFp8E4M3 {M N K : UInt64} (a : @& T #[M, K]) (b : @& T #[K, N]) (scale : Float)
     (stream : CudaStream) : IO (T #[M, N])
 
+/-- `lossAndGradOut` of the attention train step (`Examples/GPU/RunMhaH100Train.lean:60-67`) as one pass:
+    `loss = 0.5 · mean((out − target)²)` (an f32 scalar tensor) and `dO = bf16((out − target) / numel)`. -/
+@[extern "lean_tyr_gpu_mse_loss_grad"]
+opaque lossAndGradOut {s : Shape} (out target : @& T s) (stream : CudaStream) : IO (T #[] × T s)
+
+/-- `sgdUpdate` (`Examples/GPU/RunMhaH100Train.lean:69-70`) fused with the bf16 cast of the next step (`:83-85`):
+    returns `(param − f32(grad) · lr, bf16 of that)`; `param` f32, `grad` bf16, bit-identical to the LibTorch chain. -/
+@[extern "lean_tyr_gpu_sgd_step"]
+opaque sgdUpdate {s : Shape} (param grad : @& T s) (lr : Float) (stream : CudaStream) : IO (T s × T s)
+
 end Tyr.GPU.GFX950
