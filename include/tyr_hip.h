@@ -86,9 +86,10 @@ int tyr_hip_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
  *
  *   q, o   : bf16 [B, Hq, N, D]      k, v : bf16 [B, Hkv, N, D], Hq % Hkv == 0
  *   window : 0 = none; > 0 requires causal != 0
- *   kv_lens: device int32 [B] (valid key count of each sequence, clamped to [1, N]) or NULL.
+ *   kv_lens: device int32 [B] (valid key count of each sequence, clamped to [0, N]) or NULL.
  *            Keys at or beyond it are masked; rows of padded queries are still written
- *            (a row that sees no key at all gets O = 0, LSE = -inf).
+ *            (a row that sees no key at all -- every row of a sequence of length 0 -- gets
+ *            O = 0, LSE = -inf; LibTorch returns NaN there).
  * tyr_hip_flash_attn_fwd is this call with Hkv = Hq, window = 0, kv_lens = NULL.
  */
 int tyr_hip_flash_attn_fwd_gqa(const void* q, const void* k, const void* v, void* o, float* lse,

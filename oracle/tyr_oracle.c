@@ -181,7 +181,7 @@ void oracle_attn_fwd_f64_mask(const uint16_t* q, const uint16_t* k, const uint16
             const uint16_t* qr = q + (bh * N + i) * D;
             int64_t len = kv_lens ? kv_lens[b] : N;
             if (len > N) len = N;
-            if (len < 1) len = 1;
+            if (len < 0) len = 0;                      /* an empty sequence: O = 0, LSE = -inf, no gradients */
             int64_t jhi = causal ? (i + 1 < len ? i + 1 : len) : len;       /* exclusive */
             int64_t jlo = window > 0 ? (i - window + 1 > 0 ? i - window + 1 : 0) : 0;
             float* orow = o + (bh * N + i) * D;
@@ -300,7 +300,7 @@ void oracle_attn_bwd_f64_mask(const uint16_t* q, const uint16_t* k, const uint16
         const uint16_t* vh = v + bk * N * D;
         int64_t len = kv_lens ? kv_lens[b] : N;
         if (len > N) len = N;
-        if (len < 1) len = 1;
+        if (len < 0) len = 0;                      /* an empty sequence: O = 0, LSE = -inf, no gradients */
         double* dka = (double*)calloc((size_t)(N * D), sizeof(double));
         double* dva = (double*)calloc((size_t)(N * D), sizeof(double));
         double* p = (double*)malloc(sizeof(double) * (size_t)N);

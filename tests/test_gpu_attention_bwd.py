@@ -85,7 +85,7 @@ def test_flash_attn_bwd_grouped_window_lengths(gpu, B, Hq, Hkv, N, D, mode):
     sc = 1 / math.sqrt(D)
     causal = "noncausal" not in mode
     window = 70 if mode in ("window", "all") else 0
-    lens = ([N, 1, N // 2, 65, N, 3, N - 1, 128][:B]) if mode in ("lens", "lens_noncausal", "all") else None
+    lens = ([N, 0, N // 2, 65, N, 3, N - 1, 128][:B]) if mode in ("lens", "lens_noncausal", "all") else None
     lens_d = None if lens is None else torch.tensor(lens, dtype=torch.int32, device="cuda")
     qd, kd, vd, gd = (t.cuda() for t in (q, k, v, g))
     o, lse = gpu.flash_attn_fwd(qd, kd, vd, causal=causal, scale=sc, window=window, kv_lens=lens_d)

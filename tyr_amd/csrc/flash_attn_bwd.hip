@@ -164,10 +164,10 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
     const size_t head_off = (size_t)bh * N * D;
     const uint16_t* Kh = Kp + (size_t)kvbh * N * D;
     const uint16_t* Vh = Vp + (size_t)kvbh * N * D;
-    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    const int Nk = (EXT && kv_lens != nullptr) ? max(0, min(N, kv_lens[bh / Hq])) : N;
     const uint8_t* km = (EXT && key_mask != nullptr) ? key_mask + (size_t)(bh / Hq) * N : nullptr;
     const int kv_end = CAUSAL ? min(Nk, q0 + C::BM) : Nk;
-    const int nkv_abs = (kv_end + C::BN - 1) / C::BN;
+    const int nkv_abs = max(1, (kv_end + C::BN - 1) / C::BN);   // a sequence without keys still walks one (fully masked) tile
     const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / C::BN, nkv_abs - 1) : 0;
     const int nkv = nkv_abs - jbase;             // tiles are numbered from jbase below
     const int qpos = qw0 + r;
@@ -373,7 +373,7 @@ __global__ __launch_bounds__(fab::THREADS, 1) void flash_attn_bwd_dkv_kernel(
     const size_t head_off = (size_t)bh * N * D;                       // of K, V, dK, dV
     const int hkv = Hq / G;
     const size_t qh0 = (size_t)(bh / hkv) * Hq + (size_t)(bh % hkv) * G;   // first query head of the group
-    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / hkv])) : N;
+    const int Nk = (EXT && kv_lens != nullptr) ? max(0, min(N, kv_lens[bh / hkv])) : N;
     // this lane's key is hidden from every query by the key mask
     const bool key_off = EXT && key_mask != nullptr && key_mask[(size_t)(bh / hkv) * N + min(kvpos, N - 1)] == 0;
 

@@ -119,12 +119,13 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint16_t* Kh = Kp + kv_head_off;
     const uint16_t* Vh = Vp + kv_head_off;
 
-    // keys at or beyond Nk are masked; with a window, query i sees keys (i - window, i]
-    const int Nk = (EXT && kv_lens != nullptr) ? max(1, min(N, kv_lens[bh / Hq])) : N;
+    // keys at or beyond Nk are masked (Nk = 0: the sequence has no keys, O = 0 and LSE = -inf); with a window,
+    // query i sees keys (i - window, i]
+    const int Nk = (EXT && kv_lens != nullptr) ? max(0, min(N, kv_lens[bh / Hq])) : N;
     // per-sequence key mask (nonzero = visible), any pattern
     const uint8_t* km = (EXT && key_mask != nullptr) ? key_mask + (size_t)(bh / Hq) * N : nullptr;
     const int kv_end = CAUSAL ? min(Nk, q0 + BM) : Nk;
-    const int nkv_abs = (kv_end + BN - 1) / BN;
+    const int nkv_abs = max(1, (kv_end + BN - 1) / BN);   // a sequence without keys still walks one (fully masked) tile
     const int jbase = (EXT && window > 0) ? min(max(0, q0 - window + 1) / BN, nkv_abs - 1) : 0;   // first tile any row sees
     const int nkv = nkv_abs - jbase;             // tiles are numbered from jbase below
 
@@ -242,6 +243,11 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
             mfma_k_group(sA, grp, kf[grp & 1]);
         }
     }
+    // Every wave has read K(0) before any wave's first tile step requests K(2) into the same stage.  (From the
+    // second step on the barrier at the end of a step separates the reads of a stage from its next request; the
+    // prologue has none of its own, and a request that is served by the L2 can land within a few hundred
+    // nanoseconds -- less than a wave can lag behind another that shares its SIMD with a second workgroup.)
+    __syncthreads();
 
     // One kv tile: softmax and P V of tile j (scores in `cur`), overlapped with the score MFMAs of
     // tile j+1 (into `nxt`).  K runs one tile ahead of V in LDS: at entry K(j+1) and V(j) are
