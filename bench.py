@@ -798,11 +798,39 @@ def wl_dsl_simple_gemm(torch, tyr, steps, warmup, cpu, parity):
     return res
 
 
+def wl_dsl_h100_gemm(torch, tyr, steps, warmup, cpu, parity):
+    """The reference's H100 bf16 GEMM surface (Tyr/GPU/Kernels/Bf16Gemm.lean:64-73: 128x256 output tile, four K slices
+    of 64, B as N x K) emitted for gfx950: a group of four waves per tile, B read from LDS by the products."""
+    from tyr_amd.dsl import kernels, runtime
+    M = N = 8192
+    K = 256                                                     # fixed by the program
+    torch.manual_seed(0)
+    a = (_normal(torch, M, K) * K ** -0.25).to(torch.bfloat16)
+    b = (_normal(torch, N, K) * K ** -0.25).to(torch.bfloat16)
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    kern = kernels.tkH100Bf16GemmFwd()
+    fn = lambda: runtime.launch(kern, [a, b, c, M, N, K], grid=(N // 256, M // 128, 1), block=(128, 1, 1))
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+    nbytes = (M * K + N * K + M * N) * 2
+    res = {"metric": "emitted GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+           "dtype": "bf16",
+           "config": {"workload": "tile-DSL program tkH100Bf16GemmFwd emitted for gfx950, bf16 x bf16 -> bf16, M=N=8192 K=256 "
+                                  "(K is fixed by the program), 128x256 tile per group of four waves",
+                      "note": f"at K = 256 the problem moves {nbytes:,} B for 34.4 GFLOP: {nbytes / (ms * 1e-3) / 1e9:.0f} GB/s"},
+           "roofline": _mfma_roofline(torch, "mfma_bf16", "tkH100Bf16GemmFwd (emitted)", tf, None)}
+    if parity:
+        ref = a[:256].float() @ b.float().t()
+        rel = float((c[:256].float() - ref).norm() / ref.norm())
+        res["parity"] = _parity(tol=1e-2, rel_fro=rel, sample="first 256 rows of C against an f32 product of the rounded operands")
+    return res
+
+
 WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "mha_train_step": wl_train_step,
              "mha_train_step_ref_shape": wl_train_step_ref_shape, "gqa_decode": wl_decode, "gqa_decode_split4": wl_decode_split4,
              "gqa_decode_small_batch": wl_decode_small_batch, "gemm_bf16": wl_gemm_bf16,
              "gemm_fp8": wl_gemm_fp8, "decode_step": wl_decode_step, "rope_fwd": wl_rope, "layernorm_residual": wl_layernorm,
-             "copy_kernel": wl_copy_kernel, "dsl_simple_gemm": wl_dsl_simple_gemm}
+             "copy_kernel": wl_copy_kernel, "dsl_simple_gemm": wl_dsl_simple_gemm, "dsl_h100_gemm": wl_dsl_h100_gemm}
 CALIBRATION = {"copy_1gib": wl_copy, "mfma_sustain_bf16": wl_mfma_bf16, "mfma_sustain_fp8": wl_mfma_fp8}
 
 

@@ -294,7 +294,11 @@ def test_programs_too_large_for_one_wave_are_run_by_a_wave_group():
     text = dsl.emit_kernel(g)
     assert "__launch_bounds__(256)" in text and "const int tyr_wave = wave::index();" in text
     assert "rt<float, 32, 256, layout::row>" in text and "rt<float, 128, 256" not in text
-    assert "wave::load_part(" in text and "wave::store_part(" in text and ", tyr_wave * 32);" in text
+    # global <-> LDS moves are shared out among the waves, the loop's tiles one iteration ahead
+    assert "wave::gload_part(" in text and "wave::sstore_part(" in text and "wave::store_part(" in text
+    assert ", tyr_wave * 32);" in text
+    plain = dsl.emit_kernel(g, prefetch_global_loads=False)
+    assert "wave::load_part(" in plain and "gload_part" not in plain
     assert re.search(r"wave::mma_ABt\(v\d+, v\d+, v14, v\d+\);", text)           # B operand = the LDS tile itself
     # a row slice stored to LDS is followed by a barrier before the group reads the whole tile
     i = text.index("wave::store(v17")

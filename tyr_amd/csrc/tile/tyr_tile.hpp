@@ -283,9 +283,44 @@ __device__ __forceinline__ void store_add(const gl<float>& dst, const sv<float, 
 }
 
 // ---------------------------------------------------------------- LDS <-> registers
+namespace detail {
+// The four slots 4q .. 4q+3 of a ROW tile are four consecutive columns of one row: one 4-element access.
+template <typename T> struct quad { T v[4]; } __attribute__((aligned(sizeof(T) * 4 <= 16 ? sizeof(T) * 4 : 16)));
+template <typename T, int RS, int R, int C>
+__device__ __forceinline__ void load_rows(rt<T, RS, C, layout::row>& dst, const st<T, R, C>& src, int row0) {
+#pragma unroll
+    for (int rb = 0; rb < RS / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const quad<T> v = *reinterpret_cast<const quad<T>*>(src.at(row0 + 32 * rb + lr(), 32 * cb + 8 * q + 4 * lg()));
+#pragma unroll
+                for (int x = 0; x < 4; ++x) dst.data[rb][cb][4 * q + x] = v.v[x];
+            }
+}
+template <typename T, int RS, int R, int C>
+__device__ __forceinline__ void store_rows(st<T, R, C>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
+#pragma unroll
+    for (int rb = 0; rb < RS / 32; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                quad<T> v;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) v.v[x] = src.data[rb][cb][4 * q + x];
+                *reinterpret_cast<quad<T>*>(dst.at(row0 + 32 * rb + lr(), 32 * cb + 8 * q + 4 * lg())) = v;
+            }
+}
+}  // namespace detail
 template <typename T, int R, int C, layout L>
 __device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src) {
     typedef rt<T, R, C, L> RT;
+    if constexpr (L == layout::row) {
+        detail::load_rows(dst, src, 0);
+        return;
+    }
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *src.at(row_of<L>(rb, s), col_of<L>(cb, s));
 }
 // COL tiles of 2-byte elements: a lane wants 4 consecutive rows of one column per slot group, which is
@@ -308,6 +343,11 @@ __device__ __forceinline__ void load(rt<bf16, R, C, layout::col>& dst, const st<
 template <typename T, int R, int C, layout L>
 __device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, R, C, L>& src) {
     typedef rt<T, R, C, L> RT;
+    if constexpr (L == layout::row) {
+        detail::store_rows(dst, src, 0);
+        wave_fence();
+        return;
+    }
     TYR_TILE_FOR_BLOCKS(RT) *dst.at(row_of<L>(rb, s), col_of<L>(cb, s)) = src.data[rb][cb][s];
     wave_fence();
 }
@@ -757,18 +797,44 @@ __device__ __forceinline__ void store_part(const gl<T>& dst, const st<T, R, C>& 
         *reinterpret_cast<u32x4*>(dst.at(at.b, at.d, at.r + r, at.c + c)) = *reinterpret_cast<const u32x4*>(src.at(r, c));
     }
 }
+// The two halves of load_part with the pieces a lane moves held in registers in between (wave `part` of W
+// takes pieces part*64 + lane, + 64 W, ...): the next iteration's tile is requested before the products of
+// the current one.
+template <typename T, int R, int C, int W>
+struct gfrag_part {
+    static constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC, N = R * CPR / (64 * W);
+    static_assert(C % VEC == 0 && (R * CPR) % (64 * W) == 0, "the waves share the tile's 16-byte pieces evenly");
+    u32x4 v[N];
+};
+template <typename T, int R, int C, int W>
+__device__ __forceinline__ void gload_part(gfrag_part<T, R, C, W>& dst, const gl<T>& src, coord at, int part) {
+    typedef gfrag_part<T, R, C, W> F;
+#pragma unroll
+    for (int k = 0; k < F::N; ++k) {
+        const int idx = part * 64 + lane() + 64 * W * k, r = idx / F::CPR, c = (idx % F::CPR) * F::VEC;
+        dst.v[k] = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
+    }
+}
+template <typename T, int R, int C, int W>
+__device__ __forceinline__ void sstore_part(st<T, R, C>& dst, const gfrag_part<T, R, C, W>& src, int part) {
+    typedef gfrag_part<T, R, C, W> F;
+#pragma unroll
+    for (int k = 0; k < F::N; ++k) {
+        const int idx = part * 64 + lane() + 64 * W * k, r = idx / F::CPR, c = (idx % F::CPR) * F::VEC;
+        *reinterpret_cast<u32x4*>(dst.at(r, c)) = src.v[k];
+    }
+    wave_fence();
+}
 // a wave's row slice of an LDS tile / vector <-> registers
 template <typename T, int RS, int R, int C>
 __device__ __forceinline__ void load(rt<T, RS, C, layout::row>& dst, const st<T, R, C>& src, int row0) {
-    typedef rt<T, RS, C, layout::row> RT;
     static_assert(RS <= R, "a slice is no taller than its tile");
-    TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *src.at(row0 + row_of<layout::row>(rb, s), col_of<layout::row>(cb, s));
+    detail::load_rows(dst, src, row0);
 }
 template <typename T, int RS, int R, int C>
 __device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
-    typedef rt<T, RS, C, layout::row> RT;
     static_assert(RS <= R, "a slice is no taller than its tile");
-    TYR_TILE_FOR_BLOCKS(RT) *dst.at(row0 + row_of<layout::row>(rb, s), col_of<layout::row>(cb, s)) = src.data[rb][cb][s];
+    detail::store_rows(dst, src, row0);
     wave_fence();
 }
 template <typename T, int NS, int N>

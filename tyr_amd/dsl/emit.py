@@ -489,7 +489,7 @@ class _Emitter:
         self.group = self.waves > 1
         self.dirty: set = set()          # LDS objects written in shares by the group since the last barrier
         # request the next iteration's global tiles of a loop before the work of the current one
-        self.prefetch_global_loads = prefetch_global_loads and not self.group and not self.streamed
+        self.prefetch_global_loads = prefetch_global_loads
         # LDS tiles with disjoint live ranges share storage
         # (only where that asks for no barrier the program does not already have)
         self.lds = lds_plan(kernel) if share_lds else {}
@@ -639,9 +639,6 @@ class _Emitter:
             return f"{ind}wave::sync();\n"
         if op in ("forLoop", "forLoopVal"):
             hi = f"{s.hi}" if op == "forLoop" else f"(int){I(s.hi)}"
-            pre = self.prefetchable(s) if self.prefetch_global_loads else []
-            if pre:
-                return self.prefetched_loop(s, hi, pre, ind)
             if self.group:                               # what the back edge may bring in, to a fixed point
                 entry = set(self.dirty)
                 while True:
@@ -650,6 +647,9 @@ class _Emitter:
                         break
                     entry = end
                 self.dirty = set(entry)
+            pre = self.prefetchable(s) if self.prefetch_global_loads else []
+            if pre:
+                return self.prefetched_loop(s, hi, pre, ind)
             return (f"{ind}for (int {I(s.v)} = {s.lo}; {I(s.v)} < {hi}; ++{I(s.v)}) {{\n" + self.body(s.body, ind + "  ") +
                     f"{ind}}}\n")
         if op == "ifStmt":
@@ -717,7 +717,14 @@ class _Emitter:
             out.append(t)
         # a tile loaded twice in the body, or written by another statement, keeps the plain form
         written = [getattr(t, "dst", None) for t in inner if t not in out]
-        return [t for t in out if t.dst not in written and sum(1 for u in out if u.dst == t.dst) == 1]
+        out = [t for t in out if t.dst not in written and sum(1 for u in out if u.dst == t.dst) == 1]
+        if self.group:                                   # the waves share a tile's 16-byte pieces evenly, or not at all
+            def even(t):
+                d = self.info[t.dst]
+                return (d.rows * d.cols * _DTYPE_BYTES[d.dtype] // 16) % (64 * self.waves) == 0
+            if not all(even(t) for t in out):
+                return []
+        return out
 
     def prefetched_loop(self, loop: Stmt, hi: str, pre, ind: str) -> str:
         I = lambda v: v.ident
@@ -727,12 +734,17 @@ class _Emitter:
             tile = self.info[t.dst]
             at = (f"coord{{(int){I(t.coordB)}, (int){I(t.coordD)}, (int){I(t.coordR)} * {tile.rows}, "
                   f"(int){I(t.coordC)} * {tile.cols}}}")
+            if self.group:
+                return f"{ind2}wave::gload_part({frag[id(t)]}, {I(t.src)}, {at}, tyr_wave);\n"
             return f"{ind2}wave::gload({frag[id(t)]}, {I(t.src)}, {at});\n"
 
         out = f"{ind}// the global tiles of iteration i+1 are requested while iteration i computes\n"
         for t in pre:
             tile = self.info[t.dst]
-            out += f"{ind}wave::gfrag<{_cpp_type(tile.dtype)}, {tile.rows}, {tile.cols}> {frag[id(t)]};\n"
+            if self.group:
+                out += f"{ind}wave::gfrag_part<{_cpp_type(tile.dtype)}, {tile.rows}, {tile.cols}, {self.waves}> {frag[id(t)]};\n"
+            else:
+                out += f"{ind}wave::gfrag<{_cpp_type(tile.dtype)}, {tile.rows}, {tile.cols}> {frag[id(t)]};\n"
         out += f"{ind}if ({loop.lo} < {hi}) {{\n{ind}  const int {I(loop.v)} = {loop.lo};\n"
         out += "".join(request(t, ind + "  ") for t in pre) + f"{ind}}}\n"
         out += f"{ind}for (int {I(loop.v)} = {loop.lo}; {I(loop.v)} < {hi}; ++{I(loop.v)}) {{\n"
@@ -743,13 +755,18 @@ class _Emitter:
         placed = False
         remaining = len(pre)
         for t in loop.body:
-            if id(t) in self.barrier_before:
-                out += f"{ind2}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
             if id(t) in frag:
-                out += f"{ind2}wave::sstore({I(t.dst)}, {frag[id(t)]});\n"
+                if id(t) in self.barrier_before:
+                    out += f"{ind2}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
+                    self.dirty = set()
+                if self.group:
+                    out += f"{ind2}wave::sstore_part({I(t.dst)}, {frag[id(t)]}, tyr_wave);\n"
+                    self.dirty.add(t.dst)
+                else:
+                    out += f"{ind2}wave::sstore({I(t.dst)}, {frag[id(t)]});\n"
                 remaining -= 1
                 continue
-            out += self.stmt(t, ind2)
+            out += self.one(t, ind2)
             if not placed and remaining == 0 and t.op == "sync":
                 out += nxt
                 placed = True
@@ -757,25 +774,28 @@ class _Emitter:
             out += nxt
         return out + f"{ind}}}\n"
 
-    def body(self, stmts, ind: str) -> str:
+    def one(self, s: Stmt, ind: str) -> str:
+        """A statement with the barriers it needs in front of it."""
         out = ""
-        for s in stmts:
-            if id(s) in self.barrier_before:
-                out += f"{ind}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
+        if id(s) in self.barrier_before:
+            out += f"{ind}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
+            self.dirty = set()
+        if self.group:
+            reads, writes = self._group_rw(s)
+            if reads & self.dirty:
+                out += f"{ind}wave::sync();  // inserted: the other waves' shares of a shared tile are read below\n"
                 self.dirty = set()
-            if self.group:
-                reads, writes = self._group_rw(s)
-                if reads & self.dirty:
-                    out += f"{ind}wave::sync();  // inserted: the other waves' shares of a shared tile are read below\n"
-                    self.dirty = set()
-                if s.op == "sync":
-                    self.dirty = set()
-                out += self.stmt(s, ind)
-                if s.op not in ("forLoop", "forLoopVal", "ifStmt"):
-                    self.dirty |= writes
-            else:
-                out += self.stmt(s, ind)
+            if s.op == "sync":
+                self.dirty = set()
+            out += self.stmt(s, ind)
+            if s.op not in ("forLoop", "forLoopVal", "ifStmt"):
+                self.dirty |= writes
+        else:
+            out += self.stmt(s, ind)
         return out
+
+    def body(self, stmts, ind: str) -> str:
+        return "".join(self.one(s, ind) for s in stmts)
 
     # ------------------------------------------------------------------ wave groups: who reads whose share
     def _group_rw(self, s: Stmt):
