@@ -71,7 +71,8 @@ template <int D, bool CAUSAL, bool EXT>
 __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp, const uint16_t* __restrict__ Vp,
     uint16_t* __restrict__ O, float* __restrict__ LSE, int BH, int N, int ntq, float scale_log2,
-    int Hq, int G, int window, const int* __restrict__ kv_lens, const uint8_t* __restrict__ key_mask, int pair) {
+    int Hq, int G, int window, const int* __restrict__ kv_lens, const uint8_t* __restrict__ key_mask, int pair,
+    int total_ids) {
     using namespace fa;
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -87,30 +88,44 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // query heads times ntq tiles share one K/V; the G heads of a tile are adjacent.
     // With `pair` (causal) a workgroup handles query tile ntq-1-tr and then tile tr: every
     // workgroup does the same amount of work and there are half as many of them to start.
+    // A workgroup is persistent: the launch has at most two workgroups per CU, and workgroup p walks the job ids
+    // p, p + gridDim.x, ... (gridDim.x is a multiple of 8, so all of them belong to its XCD).  The hand-over from a
+    // job's last tile to the next job's first one is the hand-over between the two tiles of a pair: no dispatch gap,
+    // and the next tile's K(0), K(1) and Q are requested under the end of the current one.
     const int ntr = pair ? (ntq + 1) / 2 : ntq;  // tile ranks per head
-    int bh, tr, kvbh;
-    {
-        const int id = blockIdx.x;
+    auto decode = [&](int id, int& bh_, int& tr_, int& kvbh_) {
         const int ngroups = BH / G;              // B * Hkv
         if ((ngroups & 7) == 0) {
             const int xcd = id & 7, slot = id >> 3;
             const int per_group = G * ntr;
-            kvbh = (slot / per_group) * 8 + xcd;
+            kvbh_ = (slot / per_group) * 8 + xcd;
             const int within = slot % per_group;
-            tr = within / G;
+            tr_ = within / G;
             const int hkv = Hq / G;
-            bh = (kvbh / hkv) * Hq + (kvbh % hkv) * G + within % G;
+            bh_ = (kvbh_ / hkv) * Hq + (kvbh_ % hkv) * G + within % G;
         } else {
-            bh = id / ntr;
-            tr = id % ntr;
-            kvbh = (bh / Hq) * (Hq / G) + (bh % Hq) / G;
+            bh_ = id / ntr;
+            tr_ = id % ntr;
+            kvbh_ = (bh_ / Hq) * (Hq / G) + (bh_ % Hq) / G;
         }
-    }
-    const int npass = (pair && ntq - 1 - tr != tr) ? 2 : 1;
+    };
     bf16x8 qf[C::KSTEPS];                        // Q^T fragments: lane holds row qw0+r, columns 16i + 8g + [0,8)
     bool preloaded = false;                      // this tile's K(0), K(1) and Q were requested by the previous one
+    for (int id = blockIdx.x; id < total_ids; id += gridDim.x) {
+    int bh, tr, kvbh;
+    decode(id, bh, tr, kvbh);
+    const int npass = (pair && ntq - 1 - tr != tr) ? 2 : 1;
     for (int pass = 0; pass < npass; ++pass) {
     const int qt = CAUSAL ? (pass == 0 ? ntq - 1 - tr : tr) : tr;
+    // what this workgroup runs after this tile: the pair's second tile, or the first tile of its next job
+    bool has_next = pass + 1 < npass;
+    int n_bh = bh, n_kvbh = kvbh, n_qt = tr;
+    if (!has_next && id + (int)gridDim.x < total_ids) {
+        int n_tr;
+        decode(id + (int)gridDim.x, n_bh, n_tr, n_kvbh);
+        n_qt = CAUSAL ? ntq - 1 - n_tr : n_tr;
+        has_next = true;
+    }
     const int q0 = qt * BM;
     const int qw0 = q0 + w * 32;                 // first query row of this wave
     const size_t head_off = (size_t)bh * N * D;
@@ -143,6 +158,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     const uint32_t head_bytes = (uint32_t)N * D * 2u;
     const u32x4 k_rsrc = make_raw_rsrc(Kh, head_bytes);
     const u32x4 v_rsrc = make_raw_rsrc(Vh, head_bytes);
+    const u32x4 nk_rsrc = make_raw_rsrc(Kp + (size_t)n_kvbh * N * D, head_bytes);     // K of the tile after this one
     // Tiles go from global memory straight into LDS (no register staging).  One load instruction
     // of a wave fills 1 KiB of LDS linearly (lane i -> 16 bytes at base + 16 i); the swizzle is
     // applied on the global side: the lane fetches the chunk that belongs at its LDS position.
@@ -162,6 +178,10 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     auto issue_k = [&](int stage, int j0) {
         const uint32_t dst = wave_dst + (uint32_t)stage * C::K_TILE;
         load_global_to_lds_16xN<C::PER_THREAD>(k_rsrc, dst, gk_voff, j0 * C::ROW);
+    };
+    auto issue_k_next = [&](int stage, int j0) {
+        const uint32_t dst = wave_dst + (uint32_t)stage * C::K_TILE;
+        load_global_to_lds_16xN<C::PER_THREAD>(nk_rsrc, dst, gk_voff, j0 * C::ROW);
     };
     auto issue_v = [&](int stage, int j0) {
         const uint32_t dst = wave_dst + C::V_BASE + (uint32_t)stage * C::V_TILE;
@@ -198,7 +218,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // The second tile of a pair starts under the end of the first: its K(0), K(1) are requested
     // in the first tile's last two steps (stage parity needs an even tile count), its Q rows
     // before the first tile's output is written.
-    const bool overlap_next = pass + 1 < npass && (nkv & 1) == 0;
+    const bool overlap_next = has_next && (nkv & 1) == 0 && !(EXT && window > 0);
     // number of kv tiles that intersect this wave's visible region
     const int nkv_w = CAUSAL ? min(nkv, (qw0 + 31) / BN + 1 - jbase) : nkv;
 
@@ -258,7 +278,8 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
         // a CU do not all queue on the texture path at once.
         // In the last two steps of the first tile of a pair the freed K stages take K(0) and K(1) of
         // the second tile (a full one, >= 2 kv tiles, starting from key 0).
-        if (j + 2 < nkv || overlap_next) issue_k(j & 1, j + 2 < nkv ? j0 + 2 * BN : (j + 2 - nkv) * BN);
+        if (j + 2 < nkv) issue_k(j & 1, j0 + 2 * BN);
+        else if (overlap_next) issue_k_next(j & 1, (j + 2 - nkv) * BN);
         if (j >= nkv_w && j + 1 < nkv) issue_v((j + 1) & 1, j0 + BN);
 
         if (j < nkv_w) {
@@ -378,7 +399,12 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // scratch in the V stages (dead after the last barrier; the K stages may already be filling for
     // the second tile of a pair) so that global stores are 16 bytes per lane along rows.  Rows are
     // unpadded; 16-byte chunks are XOR-swizzled by row.
-    if (overlap_next) load_q(tr * BM + w * 32);
+    if (overlap_next) {
+        const int qrow = min(n_qt * BM + w * 32 + r, N - 1);
+        const uint16_t* qp = Q + (size_t)n_bh * N * D + (size_t)qrow * D + g * 8;
+#pragma unroll
+        for (int i = 0; i < C::KSTEPS; ++i) qf[i] = __builtin_bit_cast(bf16x8, ld_global_16(qp + i * 16));
+    }
     const float ltot = sum_xor32(lsum);
     const float inv = (!EXT || ltot > 0.0f) ? 1.0f / ltot : 0.0f;    // EXT: a row that saw no key gives 0
     {
@@ -410,6 +436,7 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     __syncthreads();                             // the scratch is read; the stages may be refilled
     preloaded = overlap_next;
     }
+    }
 }
 
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
@@ -422,7 +449,15 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
     const int ntq = (N + BM - 1) / BM;
     const bool ext = window > 0 || kv_lens != nullptr || key_mask != nullptr;
     const int pair = (causal && window <= 0 && ntq > 1) ? 1 : 0;   // lengths and key masks keep tile 0 starting at key 0
-    dim3 grid((unsigned)(BH * (pair ? (ntq + 1) / 2 : ntq))), block(THREADS);
+    const int total_ids = BH * (pair ? (ntq + 1) / 2 : ntq);
+    // two workgroups fit a CU (registers, and 64 KB of LDS each at D = 128): that many persistent workgroups
+    static const int resident = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return 2 * cus / 8 * 8;
+    }();
+    dim3 grid((unsigned)(total_ids < resident ? total_ids : resident)), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
     auto Kp = static_cast<const uint16_t*>(k);
@@ -435,7 +470,7 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DD>::LDS);                           \
         if (attr != hipSuccess) return -1;                                                       \
         hipLaunchKernelGGL((flash_attn_fwd_kernel<DD, CC, EE>), grid, block, Cfg<DD>::LDS, stream, \
-                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens, key_mask, pair); \
+                           Qp, Kp, Vp, Op, lse, BH, N, ntq, scale_log2, Hq, G, window, kv_lens, key_mask, pair, total_ids); \
     } while (0)
 #define TYR_FA_PICK(DD)                                                                          \
     do {                                                                                         \
