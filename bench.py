@@ -47,7 +47,7 @@ PEAK = {"mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "hbm": 8000.0}   # TFLOP/s, TFL
 # read for the 1 GiB copy of --workload copy_1gib (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the raw
 # figures are kept as text under profiles/.
 BWD_KERNELS = "flash_attn_bwd_dq_kernel<128,true> + flash_attn_bwd_dkv_kernel<128,true>"
-TRAFFIC = {"attn_fwd_causal": 1_073_162_240 + 272_629_760, "gqa_decode": 1_090_820_096 + 270_336,
+TRAFFIC = {"attn_fwd_causal": 1_119_610_880 + 274_726_912, "gqa_decode": 1_090_820_096 + 270_336,
            "gemm_bf16": 202_589_594 + 33_554_432, "gemm_fp8": 810_477_568 + 136_314_880,
            # both backward kernels: dQ (1,713,229,824 + 276,824,064) + dK/dV (1,082,617,856 + 536,870,912)
            "attn_bwd_causal": 1_647_249_408 + 276_824_064 + 1_082_636_288 + 536_870_912,
@@ -57,7 +57,7 @@ TRAFFIC = {"attn_fwd_causal": 1_073_162_240 + 272_629_760, "gqa_decode": 1_090_8
            "decode_rope_append_kernel + gqa_decode_split_kernel<8>": 423_680 + 393_216 + 1_090_152_448 + 270_336,
            "gqa_decode_split4": 1_085_655_040 + 2_228_224 + 2_403_328 + 294_912,       # split pass + combine pass
            "gqa_decode_small_batch": 542_947_328 + 589_824 + 601_088 + 36_864,
-           "dsl_simple_gemm": 77_063_987 + 268_435_456}
+           "dsl_simple_gemm": 77_063_987 + 268_435_456, "dsl_h100_gemm": 37_877_146 + 134_217_728}
 
 
 def _events(torch, n):
@@ -818,7 +818,7 @@ def wl_dsl_h100_gemm(torch, tyr, steps, warmup, cpu, parity):
            "config": {"workload": "tile-DSL program tkH100Bf16GemmFwd emitted for gfx950, bf16 x bf16 -> bf16, M=N=8192 K=256 "
                                   "(K is fixed by the program), 128x256 tile per group of four waves",
                       "note": f"at K = 256 the problem moves {nbytes:,} B for 34.4 GFLOP: {nbytes / (ms * 1e-3) / 1e9:.0f} GB/s"},
-           "roofline": _mfma_roofline(torch, "mfma_bf16", "tkH100Bf16GemmFwd (emitted)", tf, None)}
+           "roofline": _mfma_roofline(torch, "mfma_bf16", "tkH100Bf16GemmFwd (emitted)", tf, TRAFFIC["dsl_h100_gemm"])}
     if parity:
         ref = a[:256].float() @ b.float().t()
         rel = float((c[:256].float() - ref).norm() / ref.norm())
