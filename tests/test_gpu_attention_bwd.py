@@ -175,3 +175,16 @@ def test_flash_attn_bwd_arbitrary_key_mask(gpu, B, Hq, Hkv, N, D, causal):
     assert float(dk.cpu().float()[hidden].abs().max()) == 0.0 and float(dv.cpu().float()[hidden].abs().max()) == 0.0
     if causal:                                            # left-padded rows that saw no key: dQ = 0
         assert float(dq[1, :, : N // 3].float().abs().max()) == 0.0
+
+
+def test_flash_attn_backward_is_reproducible_over_many_launches(gpu):
+    # Every output element is written once by one workgroup (no atomics), so launches must agree bit for bit; a
+    # write-after-read race on an LDS stage would show up here as a few differing rows in some launches.
+    B, H, N, D = 8, 16, 4096, 128
+    torch.manual_seed(12)
+    q, k, v, g = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(4))
+    o, lse = gpu.flash_attn_fwd(q, k, v, causal=True)
+    first = gpu.flash_attn_bwd(q, k, v, o, lse, g, causal=True)
+    for _ in range(5):
+        again = gpu.flash_attn_bwd(q, k, v, o, lse, g, causal=True)
+        assert all(torch.equal(a, b) for a, b in zip(first, again))

@@ -315,3 +315,19 @@ def test_fp8_gemm_e4m3_output(gpu, trans_b):
         # to a small value carries an absolute error of up to ~16 in accumulator units)
         assert bool((d <= want.float().abs() * 2.0 ** -3 + 2.0 ** -9 + 16.0 * scale).all())
         assert float(c.float().abs().max()) <= 448.0 and not bool(torch.isnan(c.float()).any())
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gemms_are_reproducible_over_many_launches(gpu, trans_b):
+    # bit-identical results launch after launch at sizes with many slices and several tiles per CU
+    torch.manual_seed(13)
+    a = (torch.randn(4096, 4096, device="cuda") * 0.125).to(torch.bfloat16)
+    b = (torch.randn(4096, 4096, device="cuda") * 0.125).to(torch.bfloat16)
+    first = gpu.gemm_bf16(a, b, trans_b=trans_b)
+    aq, sa = gpu.quantize_e4m3(torch.randn(8192, 4096, device="cuda"))
+    bq, sb = gpu.quantize_e4m3(torch.randn(4096, 8192, device="cuda"))
+    bqb = bq.t().contiguous() if trans_b else bq
+    first8 = gpu.gemm_fp8(aq, bqb, sa, sb, trans_b=trans_b)
+    for _ in range(8):
+        assert torch.equal(gpu.gemm_bf16(a, b, trans_b=trans_b), first)
+        assert torch.equal(gpu.gemm_fp8(aq, bqb, sa, sb, trans_b=trans_b), first8)
