@@ -864,8 +864,19 @@ def main() -> int:
 
     if args.workload in CALIBRATION:
         args.no_extra = True
-    head = {**WORKLOADS, **CALIBRATION}[args.workload](torch, tyr_amd, args.steps, args.warmup, not args.no_cpu,
-                                                        not args.no_parity)
+    def run(fn, steps, warmup):
+        """A failing checker or CPU leg must not take the measurement with it: the workload is then measured again
+        without them and the failure is reported in its place."""
+        try:
+            return fn(torch, tyr_amd, steps, warmup, not args.no_cpu, not args.no_parity)
+        except Exception as e:
+            if args.no_cpu and args.no_parity:
+                raise
+            r = fn(torch, tyr_amd, steps, warmup, False, False)
+            r["parity"] = {"ok": False, "error": f"checker / CPU leg failed: {type(e).__name__}: {e}"}
+            return r
+
+    head = run({**WORKLOADS, **CALIBRATION}[args.workload], args.steps, args.warmup)
     line = {
         "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "settle_ms_before_warmup": PREWARM_MS,
@@ -883,8 +894,7 @@ def main() -> int:
                 continue
             torch.cuda.empty_cache()
             try:
-                r = fn(torch, tyr_amd, max(10, args.steps // 2), max(3, args.warmup // 2), not args.no_cpu,
-                       not args.no_parity)
+                r = run(fn, max(10, args.steps // 2), max(3, args.warmup // 2))
             except Exception as e:                      # a side workload must not take the headline line with it
                 r = {"error": f"{type(e).__name__}: {e}"}
             r["workload"] = name
