@@ -255,9 +255,9 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
         if (j < nkv_w) {
             const unsigned char* Kt = lds + (j & 1) * C::TILE;
             const unsigned char* Vt = Kt + C::V_BASE;
-            // The two 32-row sub-tiles of the tile are staggered so that the vector work of one has
-            // matrix work of the other next to it in program order: scores of T=0, then scores of T=1
-            // beside the exponentials of T=0, then the dQ products of T=0 beside the exponentials of T=1.
+            // The two 32-row sub-tiles of the tile are taken one after the other (scores, probabilities, dQ
+            // products): only one sub-tile's scores are live, which leaves the registers the fragment read-ahead
+            // needs; the other wave of the SIMD has matrix work while this one does its exponentials.
             f32x16 s[2], dp[2];
             bf16x8 dsf[4];
             // the tile's 64 key-mask bytes as one word (bit r set: kv row j0 + r is hidden): one byte per
@@ -269,12 +269,26 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             auto scores = [&](int T) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
+                // Fragments are read one k-step ahead of the products that take them, and the scheduling barriers keep
+                // that order: left to itself the compiler, at its register limit, puts every read right in front of its
+                // product and the wave waits out the LDS latency 48 times per tile.
+                constexpr int DEPTH = 1;
+                bf16x8 ka[DEPTH + 1], va[DEPTH + 1];
+#pragma unroll
+                for (int i = 0; i < DEPTH; ++i) {
+                    ka[i] = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
+                    va[i] = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
+                }
 #pragma unroll
                 for (int i = 0; i < C::KSTEPS; ++i) {
-                    const bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
-                    s[T] = mfma_32x32x16_bf16(ka, qf[i], s[T]);
-                    const bf16x8 va = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
-                    dp[T] = mfma_32x32x16_bf16(va, dof[i], dp[T]);
+                    if (i + DEPTH < C::KSTEPS) {
+                        ka[(i + DEPTH) % (DEPTH + 1)] = *reinterpret_cast<const bf16x8*>(Kt + row_off[i + DEPTH] + T * 32 * C::ROW);
+                        va[(i + DEPTH) % (DEPTH + 1)] = *reinterpret_cast<const bf16x8*>(Vt + row_off[i + DEPTH] + T * 32 * C::ROW);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    s[T] = mfma_32x32x16_bf16(ka[i % (DEPTH + 1)], qf[i], s[T]);
+                    dp[T] = mfma_32x32x16_bf16(va[i % (DEPTH + 1)], dof[i], dp[T]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             };
             // mask (diagonal tiles, ragged tail), then dS^T = P^T o (dP^T - delta) packed into column-operand
@@ -308,21 +322,27 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             };
             // dQ^T += K^T dS^T for the two 16-row groups of sub-tile T
             auto accumulate = [&](int T) {
+                bf16x4 lo[2], hi[2];
+                lo[0] = ds_read_tr16(Kt + tr_lo[0] + 2 * T * 16 * C::ROW);
+                hi[0] = ds_read_tr16(Kt + tr_hi[0] + 2 * T * 16 * C::ROW);
 #pragma unroll
-                for (int c = 2 * T; c < 2 * T + 2; ++c) {
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt) {
-                        const bf16x4 lo = ds_read_tr16(Kt + tr_lo[dt] + c * 16 * C::ROW);
-                        const bf16x4 hi = ds_read_tr16(Kt + tr_hi[dt] + c * 16 * C::ROW);
-                        const bf16x8 kt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                        dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
+                for (int n = 0; n < 2 * C::DT; ++n) {          // n = (c - 2T) * DT + dt
+                    const int c = 2 * T + n / C::DT, dt = n % C::DT;
+                    if (n + 1 < 2 * C::DT) {
+                        const int c1 = 2 * T + (n + 1) / C::DT, dt1 = (n + 1) % C::DT;
+                        lo[(n + 1) & 1] = ds_read_tr16(Kt + tr_lo[dt1] + c1 * 16 * C::ROW);
+                        hi[(n + 1) & 1] = ds_read_tr16(Kt + tr_hi[dt1] + c1 * 16 * C::ROW);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bf16x8 kt = __builtin_shufflevector(lo[n & 1], hi[n & 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             };
             scores(0);
-            scores(1);
             probabilities(0);
             accumulate(0);
+            scores(1);
             probabilities(1);
             accumulate(1);
         }
