@@ -266,28 +266,31 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
             if (EXT && km != nullptr) tile_hidden = __builtin_amdgcn_ballot_w64(km[min(j0 + lane, N - 1)] == 0);
             const bool need_mask = (CAUSAL && (j0 + C::BN - 1 > qw0)) || (j0 + C::BN > Nk) ||
                                    (EXT && window > 0 && j0 < qw0 + 32 - window) || (EXT && tile_hidden != 0);
-            auto scores = [&](int T) {
+            // Fragments are read one k-step ahead of the products that take them, also across the phases of a tile (the
+            // first fragments of a phase are requested under the last products of the phase before it), and the
+            // scheduling barriers keep that order: left to itself the compiler, at its register limit, puts every read
+            // right in front of its product and the wave waits out the LDS latency 48 times per tile.
+            bf16x8 ka[2], va[2];                 // K / V row fragments of the scores phase
+            bf16x4 lo[2], hi[2];                 // transposed K fragments of the dQ phase
+            auto read_rows = [&](int T, int i, int slot) {
+                ka[slot] = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
+                va[slot] = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
+            };
+            auto read_transposed = [&](int T, int n, int slot) {      // n = (c - 2T) * DT + dt
+                const int c = 2 * T + n / C::DT, dt = n % C::DT;
+                lo[slot] = ds_read_tr16(Kt + tr_lo[dt] + c * 16 * C::ROW);
+                hi[slot] = ds_read_tr16(Kt + tr_hi[dt] + c * 16 * C::ROW);
+            };
+            auto scores = [&](int T) {           // expects the fragments of k-step 0 in slot 0
 #pragma unroll
                 for (int e = 0; e < 16; ++e) { s[T][e] = 0.0f; dp[T][e] = 0.0f; }
-                // Fragments are read one k-step ahead of the products that take them, and the scheduling barriers keep
-                // that order: left to itself the compiler, at its register limit, puts every read right in front of its
-                // product and the wave waits out the LDS latency 48 times per tile.
-                constexpr int DEPTH = 1;
-                bf16x8 ka[DEPTH + 1], va[DEPTH + 1];
-#pragma unroll
-                for (int i = 0; i < DEPTH; ++i) {
-                    ka[i] = *reinterpret_cast<const bf16x8*>(Kt + row_off[i] + T * 32 * C::ROW);
-                    va[i] = *reinterpret_cast<const bf16x8*>(Vt + row_off[i] + T * 32 * C::ROW);
-                }
 #pragma unroll
                 for (int i = 0; i < C::KSTEPS; ++i) {
-                    if (i + DEPTH < C::KSTEPS) {
-                        ka[(i + DEPTH) % (DEPTH + 1)] = *reinterpret_cast<const bf16x8*>(Kt + row_off[i + DEPTH] + T * 32 * C::ROW);
-                        va[(i + DEPTH) % (DEPTH + 1)] = *reinterpret_cast<const bf16x8*>(Vt + row_off[i + DEPTH] + T * 32 * C::ROW);
-                    }
+                    if (i + 1 < C::KSTEPS) read_rows(T, i + 1, (i + 1) & 1);
+                    else read_transposed(T, 0, 0);               // first fragment of this sub-tile's dQ phase
                     __builtin_amdgcn_sched_barrier(0);
-                    s[T] = mfma_32x32x16_bf16(ka[i % (DEPTH + 1)], qf[i], s[T]);
-                    dp[T] = mfma_32x32x16_bf16(va[i % (DEPTH + 1)], dof[i], dp[T]);
+                    s[T] = mfma_32x32x16_bf16(ka[i & 1], qf[i], s[T]);
+                    dp[T] = mfma_32x32x16_bf16(va[i & 1], dof[i], dp[T]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
@@ -321,24 +324,19 @@ __global__ __launch_bounds__(fab::THREADS, 2) void flash_attn_bwd_dq_kernel(
                 }
             };
             // dQ^T += K^T dS^T for the two 16-row groups of sub-tile T
-            auto accumulate = [&](int T) {
-                bf16x4 lo[2], hi[2];
-                lo[0] = ds_read_tr16(Kt + tr_lo[0] + 2 * T * 16 * C::ROW);
-                hi[0] = ds_read_tr16(Kt + tr_hi[0] + 2 * T * 16 * C::ROW);
+            auto accumulate = [&](int T) {       // expects the transposed fragment 0 in slot 0
 #pragma unroll
-                for (int n = 0; n < 2 * C::DT; ++n) {          // n = (c - 2T) * DT + dt
+                for (int n = 0; n < 2 * C::DT; ++n) {
                     const int c = 2 * T + n / C::DT, dt = n % C::DT;
-                    if (n + 1 < 2 * C::DT) {
-                        const int c1 = 2 * T + (n + 1) / C::DT, dt1 = (n + 1) % C::DT;
-                        lo[(n + 1) & 1] = ds_read_tr16(Kt + tr_lo[dt1] + c1 * 16 * C::ROW);
-                        hi[(n + 1) & 1] = ds_read_tr16(Kt + tr_hi[dt1] + c1 * 16 * C::ROW);
-                    }
+                    if (n + 1 < 2 * C::DT) read_transposed(T, n + 1, (n + 1) & 1);
+                    else if (T == 0) read_rows(1, 0, 0);         // first fragments of the second sub-tile's scores
                     __builtin_amdgcn_sched_barrier(0);
                     const bf16x8 kt = __builtin_shufflevector(lo[n & 1], hi[n & 1], 0, 1, 2, 3, 4, 5, 6, 7);
                     dq[dt] = mfma_32x32x16_bf16(kt, dsf[c], dq[dt]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
+            read_rows(0, 0, 0);
             scores(0);
             probabilities(0);
             accumulate(0);
