@@ -371,8 +371,12 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
         };
+        // The first MFMA row goes out before any fragment of the next k-step is requested: at the top of the loop
+        // the compiler waits for every LDS read in flight (it cannot count across the back edge), and with fresh
+        // requests in front of that wait the wave would sit out their latency once per slice.
         issue_half(st ^ 1, kt + 1, 0, 0);
-        read_pair(St, 1, 0, af[1][0], bf[1][0]); TYR_FENCE; row(0, 0); TYR_FENCE;
+        TYR_FENCE; row(0, 0); TYR_FENCE;
+        read_pair(St, 1, 0, af[1][0], bf[1][0]);
         issue_half(st ^ 1, kt + 1, 0, 1);
         read_pair(St, 1, 1, af[1][1], bf[1][1]); TYR_FENCE; row(0, 1); TYR_FENCE;
         issue_half(st ^ 1, kt + 1, 1, 0);
