@@ -2,12 +2,17 @@
 """Benchmark of the gfx950 kernel hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-parity] [--no-extra]
+                    [--details FILE]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The headline workload is the causal flash-attention forward the target is quoted on
 (bf16, B=16 H=16 N=4096 D=128); the other configurations (attention backward, GQA decode, bf16 GEMM,
 fp8 GEMM)
-are measured in the same run and reported under "other_workloads" of the single JSON line.
+are measured in the same run.  Standard output carries ONE compact JSON line (a few KB): the headline
+fields, a summary of every configuration of the benchmark under "baseline_configs" and of the remaining
+workloads under "other_workloads" (time, rate, roofline fraction, HBM traffic, parity verdict, CPU figure
+with core counts).  The full records (conventions, samples, notes) go to standard error as one JSON line
+starting with {"details": and, with --details FILE, to that file.
 
 FLOP / byte conventions (algorithmic work, fixed per configuration):
   attn_fwd_causal : 4*B*H*N^2*D / 2 FLOP (two GEMMs, causal half)           -> MFMA bf16 2.5 PFLOP/s
@@ -109,7 +114,7 @@ def sustained_peak(torch, kind):
 
     def fn():
         rc = L.tyr_hip_mfma_sustain(ops.data_ptr(), ops.numel() * ops.element_size(), dtype, wgs, iters,
-                                    sink.data_ptr(), ctypes.byref(flop), st)
+                                    sink.data_ptr(), sink.numel() * sink.element_size(), ctypes.byref(flop), st)
         assert rc == 0, rc
     _, ms = time_steps(torch, fn, 20, 5)
     _SUSTAINED[kind] = {"value": flop.value / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
@@ -174,12 +179,25 @@ def wl_attn(torch, tyr, steps, warmup, cpu, parity):
     wall, ms = time_steps(torch, fn, steps, warmup)
     flop = 4.0 * B * H * N * N * D / 2.0
     tf = flop / (ms * 1e-3) / 1e12
+    # the two launch shapes of the forward, timed alternately after the headline's timed region (same box, same run)
+    from tyr_amd import _lib
+    L = _lib.load()
+    default_shape = L.tyr_hip_flash_attn_fwd_persistent(0)
+    pair = {"per_job": [], "persistent": []}
+    for _ in range(3):
+        for name, on in (("per_job", 0), ("persistent", 1)):
+            L.tyr_hip_flash_attn_fwd_persistent(on)
+            pair[name].append(time_steps(torch, fn, steps, 2)[1])
+    L.tyr_hip_flash_attn_fwd_persistent(default_shape)
+    fn()                                            # `out` holds a launch of the default shape again
     res = {
         "metric": "attn fwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
         "dtype": "bf16",
         "config": {"workload": "causal flash-attention forward, bf16, B=16 H=16 N=4096 D=128, O + LSE",
                    "flop_convention": "4*B*H*N^2*D/2 (causal half)", "scale": "1/sqrt(128)",
-                   "inputs": "torch.manual_seed(0); Q, K, V = randn on the host in that order -> bf16 -> device"},
+                   "inputs": "torch.manual_seed(0); Q, K, V = randn on the host in that order -> bf16 -> device",
+                   "launch_shape": "persistent" if default_shape else "per_job",
+                   "launch_shapes_ms": {k_: round(sorted(v_)[1], 5) for k_, v_ in pair.items()}},
         "roofline": _mfma_roofline(torch, "mfma_bf16", "flash_attn_fwd_kernel<128,true>", tf, TRAFFIC["attn_fwd_causal"]),
     }
     if parity:
@@ -492,7 +510,9 @@ def _wl_train(torch, tyr, steps, warmup, cpu, parity, shape, causal, lr, label):
         q, k, v, loss = _train_step(torch, tyr, state[0], state[1], state[2], target, lr, causal, sc)
         state[0], state[1], state[2] = q, k, v
         losses.append(loss)
-    _, ms_torch_elementwise = time_steps(torch, fn_torch_elementwise, max(5, steps // 3), 2)
+    # The same step with LibTorch element-wise calls around the kernels is a comparison leg: it runs with the output check
+    # only, so that a profile taken with --no-parity holds the kernels of the fused step and nothing else.
+    ms_torch_elementwise = time_steps(torch, fn_torch_elementwise, max(5, steps // 3), 2)[1] if parity else None
     fstate = {"m": [t.clone() for t in init]}
     fstate["l"] = [t.to(torch.bfloat16) for t in fstate["m"]]
 
@@ -834,6 +854,26 @@ WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "mha_tr
 CALIBRATION = {"copy_1gib": wl_copy, "mfma_sustain_bf16": wl_mfma_bf16, "mfma_sustain_fp8": wl_mfma_fp8}
 
 
+# the configurations of the benchmark that run on the GPU (configuration 1 is the LibTorch-CPU plumbing case)
+BASELINE_CONFIGS = {"cfg2_gemm_bf16_4096": "gemm_bf16", "cfg3_attn_fwd_causal_b16_h16_n4096_d128": "attn_fwd_causal",
+                    "cfg4_gqa_decode_b32_hq32_hkv8_l8192": "gqa_decode", "cfg5_gemm_fp8_8192": "gemm_fp8"}
+
+
+def _summary(r):
+    """The few figures of a workload record that the one-line output carries."""
+    if "error" in r:
+        return {"workload": r["workload"], "error": r["error"][:200]}
+    roof, par, cpu = r.get("roofline") or {}, r.get("parity") or {}, r.get("cpu_baseline") or {}
+    d = {"workload": r["workload"], "ms_per_step": round(r["ms_per_step"], 5), "value": round(r["value"], 1), "unit": r["unit"],
+         "bound": roof.get("bound"), "frac": round(roof.get("frac", 0.0), 4), "traffic": roof.get("traffic"),
+         "parity_ok": par.get("ok")}
+    if "error" in par:
+        d["parity_error"] = par["error"][:160]
+    if cpu:
+        d["cpu_baseline"] = {"value": round(cpu["value"], 4), "unit": cpu["unit"], "cores": cpu["cores"]}
+    return d
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -843,6 +883,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-parity", action="store_true", help="skip the check of the outputs against the CPU checker")
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
+    ap.add_argument("--details", default=None, metavar="FILE", help="also write the full records (one JSON line) to FILE")
     ap.add_argument("--settle-ms", type=float, default=PREWARM_MS,
                     help="untimed work before the warm-up steps of every workload, in milliseconds")
     ap.add_argument("--data", default="randn", choices=["randn", "constant"],
@@ -877,18 +918,9 @@ def main() -> int:
             return r
 
     head = run({**WORKLOADS, **CALIBRATION}[args.workload], args.steps, args.warmup)
-    line = {
-        "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "settle_ms_before_warmup": PREWARM_MS,
-        "ms_per_step": round(head["ms_per_step"], 5),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
-        "data": "synthetic" if DATA == "randn" else "synthetic, every operand 0.5 (power diagnostic, not the benchmark input)",
-        "config": head["config"], "roofline": head["roofline"],
-        "parity": head.get("parity"), "cpu_baseline": head.get("cpu_baseline"), "wall_ms_per_step": round(head["wall_ms_per_step"], 5),
-        "device": info,
-    }
+    head["workload"] = args.workload
+    records = [head]
     if not args.no_extra:
-        others = []
         for name, fn in WORKLOADS.items():
             if name == args.workload:
                 continue
@@ -898,9 +930,32 @@ def main() -> int:
             except Exception as e:                      # a side workload must not take the headline line with it
                 r = {"error": f"{type(e).__name__}: {e}"}
             r["workload"] = name
-            others.append(r)
-        line["other_workloads"] = others
-    print(json.dumps(line))
+            records.append(r)
+
+    host = {"nproc": os.cpu_count(), "usable_cores": len(os.sched_getaffinity(0)), "torch_threads": torch.get_num_threads()}
+    roof = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in head["roofline"].items() if k != "sustained_how"}
+    par = head.get("parity")
+    line = {
+        "metric": head["metric"], "value": round(head["value"], 3), "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "settle_ms_before_warmup": PREWARM_MS,
+        "ms_per_step": round(head["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic" if DATA == "randn" else "synthetic, every operand 0.5 (power diagnostic, not the benchmark input)",
+        "config": head["config"], "roofline": roof,
+        "parity": None if par is None else {k: (round(v, 6) if isinstance(v, float) else v) for k, v in par.items() if k != "sample"},
+        "cpu_baseline": head.get("cpu_baseline"), "wall_ms_per_step": round(head["wall_ms_per_step"], 5),
+        "device": info, "host": host,
+    }
+    by_name = {r["workload"]: r for r in records}
+    line["baseline_configs"] = {label: _summary(by_name[name]) for label, name in BASELINE_CONFIGS.items() if name in by_name}
+    if not args.no_extra:
+        line["other_workloads"] = [_summary(r) for r in records[1:] if r["workload"] not in BASELINE_CONFIGS.values()]
+    details = json.dumps({"details": records, "device": info, "host": host})
+    if args.details:
+        with open(args.details, "w") as f:
+            f.write(details + "\n")
+    print(details, file=sys.stderr, flush=True)
+    print(json.dumps(line), flush=True)
     return 0
 
 

@@ -326,6 +326,14 @@ int tyr_hip_gemm_bf16_batched(const void* a, const void* b, void* c, uint64_t ba
  * "on" iff the environment variable TYR_HIP_GEMM_GENERAL exists when the first GEMM is launched. */
 int tyr_hip_gemm_force_general(int on);
 
+/* Launch-shape switch of the forward attention kernels (no counterpart in the reference).  A forward launch
+ * starts either one workgroup per (head, query-tile job), or -- on != 0 -- two persistent workgroups per CU
+ * that walk the jobs.  Results are bit-identical; only the timing differs (which of the two is faster depends on
+ * the shape and, by a few per cent, on the individual device).  Process-wide until changed again; the previous
+ * setting is returned.  The initial setting is "on" iff the environment variable TYR_HIP_FA_PERSISTENT is "1"
+ * when the first forward is launched. */
+int tyr_hip_flash_attn_fwd_persistent(int on);
+
 /* ---------------------------------------------------------------------------
  * FP8 E4M3 GEMM with per-tensor f32 scales, bf16 output:
  *     C = bf16( scale_a * scale_b * (Aq Bq) ),  f32 accumulation, scale in the epilogue.
@@ -386,11 +394,12 @@ int tyr_hip_sgd_step(const float* param, const void* grad, float lr, float* para
  * runners print a torch figure beside the kernel's (Examples/GPU/RunMhaH100Train.lean:217-288).
  * Every wave of `workgroups` 4-wave workgroups loads 8 operand fragments from `operands` once and
  * then issues only MFMAs (32x32x16 bf16 or 32x32x64 E4M3), `iters` rounds of 16.  *flop_per_launch
- * receives the floating-point operations of one launch.  `sink` takes 256 floats per workgroup.
+ * receives the floating-point operations of one launch.  `sink` (device memory of `sink_bytes` bytes) takes 256
+ * floats per workgroup; a smaller buffer is refused with TYR_HIP_ERR_WORKSPACE before anything is launched.
  */
 enum tyr_hip_mfma_type { TYR_HIP_MFMA_BF16 = 0, TYR_HIP_MFMA_E4M3 = 1 };
 int tyr_hip_mfma_sustain(const void* operands, size_t operand_bytes, int dtype, uint64_t workgroups,
-                         uint64_t iters, float* sink, double* flop_per_launch, void* stream);
+                         uint64_t iters, float* sink, size_t sink_bytes, double* flop_per_launch, void* stream);
 
 #ifdef __cplusplus
 }

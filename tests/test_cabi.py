@@ -52,6 +52,10 @@ def test_host_validation_needs_no_gpu():
     assert L.tyr_hip_gemm_bf16_batched(p, p, p, 70000, 8, 8, 8, 64, 64, 64, 0, None) == SHAPE
     prev = L.tyr_hip_gemm_force_general(1)
     assert L.tyr_hip_gemm_force_general(prev) == 1 and L.tyr_hip_gemm_force_general(prev) == prev
+    prev = L.tyr_hip_flash_attn_fwd_persistent(1)
+    assert L.tyr_hip_flash_attn_fwd_persistent(prev) == 1 and L.tyr_hip_flash_attn_fwd_persistent(prev) == prev
+    # the calibration loop writes 256 floats per workgroup: a smaller sink is refused before any launch
+    assert L.tyr_hip_mfma_sustain(p, 1 << 20, 0, 256, 10, p, 256 * 256 * 4 - 1, None, None) == WS
     assert L.tyr_hip_gemm_fp8(p, p, None, 16, 16, 16, 1.0, 1.0, 0, None) == NULL
     assert L.tyr_hip_gemm_fp8(p, p, p, 16, 8, 16, 1.0, 1.0, 0, None) == UNSUP
     assert L.tyr_hip_gemm_fp8_ex(p, p, p, 16, 16, 16, 1.0, None, None, 7, 0, None) == UNSUP           # unknown output type

@@ -98,18 +98,26 @@ def test_flash_attn_future_keys_do_not_leak(gpu):
     assert not torch.equal(a[:, :, 320:], b[:, :, 320:])
 
 
+@pytest.mark.parametrize("persistent", [0, 1])
 @pytest.mark.parametrize("causal", [True, False])
-def test_flash_attn_forward_is_reproducible_over_many_launches(gpu, causal):
+def test_flash_attn_forward_is_reproducible_over_many_launches(gpu, causal, persistent):
     # Regression test for a write-after-read race on the first K stage: the first tile step used to request K(2)
     # into the stage other waves were still reading K(0) from (no barrier after the prologue's scores); whether a
     # wave lost depended on timing, a few dozen waves per launch at this size.  Eight launches must agree bit for bit.
     B, H, N, D = 16, 16, 4096, 128
     torch.manual_seed(11)
     q, k, v = (torch.randn(B, H, N, D, device="cuda").to(torch.bfloat16) for _ in range(3))
-    first = gpu.flash_attn_fwd(q, k, v, causal=causal)
-    for _ in range(7):
-        o, lse = gpu.flash_attn_fwd(q, k, v, causal=causal)
-        assert torch.equal(o, first[0]) and torch.equal(lse, first[1])
+    with _persistent(persistent):
+        first = gpu.flash_attn_fwd(q, k, v, causal=causal)
+        for _ in range(7):
+            o, lse = gpu.flash_attn_fwd(q, k, v, causal=causal)
+            assert torch.equal(o, first[0]) and torch.equal(lse, first[1])
+    # values, not only agreement between launches: two heads against the double-precision checker
+    sc = 1 / math.sqrt(D)
+    for (b, h) in ((1, 2), (B - 1, H - 1)):
+        o64, lse64 = oracle.attn_fwd_f64(bits(q[b:b + 1, h:h + 1]), bits(k[b:b + 1, h:h + 1]), bits(v[b:b + 1, h:h + 1]), causal, sc)
+        assert max_abs(first[0][b, h].cpu().float(), o64[0, 0]) <= TOL
+        assert max_abs(first[1][b, h].cpu(), lse64[0, 0]) <= TOL
 
 
 def test_flash_attn_full_size_config(gpu):
@@ -140,6 +148,94 @@ def test_flash_attn_full_size_config(gpu):
     # size-independent properties: row 0 is V[0]; softmax weights reconstructed from LSE sum to one
     assert torch.equal(o[:, :, 0], v[:, :, 0])
     assert torch.equal(gpu.flash_attn_fwd(q, k, v, causal=True, scale=sc)[0], o)   # deterministic
+
+
+# ------------------------------------------- launch shape: one workgroup per job id / persistent workgroups
+
+class _persistent:
+    """Forward launches inside the block use persistent workgroups (on = 1) or one workgroup per job id (on = 0)."""
+
+    def __init__(self, on):
+        self.on = on
+
+    def __enter__(self):
+        from tyr_amd import _lib
+        self.prev = _lib.load().tyr_hip_flash_attn_fwd_persistent(int(self.on))
+
+    def __exit__(self, *exc):
+        from tyr_amd import _lib
+        _lib.load().tyr_hip_flash_attn_fwd_persistent(self.prev)
+
+
+def _mixed_lengths(B, N):
+    """Key lengths that give a persistent workgroup every kind of hand-over: full, empty, one tile or less, odd and even
+    tile counts, a ragged last tile."""
+    pool = [N, 0, 1, 64, 63, 65, 128, 192, N - 1, N // 2 + 7, 200, N]
+    return [pool[i % len(pool)] for i in range(B)]
+
+
+_MANY_JOBS_CASES = ["noncausal", "causal", "causal_lens", "noncausal_lens", "key_mask", "causal_key_mask",
+                    "gqa_causal", "gqa_noncausal", "gqa_lens_odd_groups"]
+
+
+@pytest.mark.parametrize("case", _MANY_JOBS_CASES)
+def test_flash_attn_persistent_launch_walks_many_jobs(gpu, case):
+    # More job ids than the 512 persistent workgroups of a 256-CU device, so that workgroups hand over from one job to
+    # the next (another head, another batch entry with another key length or mask, the XCD mapping of grouped queries).
+    # The persistent launch must equal the one-workgroup-per-job launch bit for bit, and sampled heads must match the
+    # double-precision checker.
+    D = 128
+    causal = "noncausal" not in case
+    lens = km = None
+    if case.startswith("gqa"):
+        B, Hq, Hkv, N = (8, 16, 4, 1280) if case != "gqa_lens_odd_groups" else (9, 12, 3, 1100)
+    elif "lens" in case or "mask" in case:
+        B, Hq, Hkv, N = 24, 8, 8, 768 if causal else 520
+    else:
+        B, Hq, Hkv, N = 12, 10, 10, 1280 if causal else 1100
+    ntq = (N + 127) // 128
+    pair = causal and ntq > 1
+    ids = B * Hq * ((ntq + 1) // 2 if pair else ntq)
+    assert ids > 512, ids
+    g = torch.Generator().manual_seed(1500 + _MANY_JOBS_CASES.index(case))
+    q = torch.randn(B, Hq, N, D, generator=g).to(torch.bfloat16)
+    k, v = (torch.randn(B, Hkv, N, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    if "lens" in case:
+        lens = _mixed_lengths(B, N)
+    if "mask" in case:
+        km = torch.rand(B, N, generator=g) < 0.7
+        km[1] = False                                   # a sequence without visible keys
+        km[2, 128:384] = False                          # whole key tiles hidden
+        km[3] = True
+        km[:, 0] |= torch.arange(B) % 2 == 0
+        km[1] = False
+    sc = 1 / math.sqrt(D)
+    kw = dict(causal=causal, scale=sc)
+    if lens is not None:
+        kw["kv_lens"] = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    if km is not None:
+        kw["key_mask"] = km.cuda()
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    with _persistent(0):
+        o0, l0 = gpu.flash_attn_fwd(qd, kd, vd, **kw)
+    with _persistent(1):
+        o1, l1 = gpu.flash_attn_fwd(qd, kd, vd, **kw)
+        o2, l2 = gpu.flash_attn_fwd(qd, kd, vd, **kw)
+    assert torch.equal(o0, o1) and torch.equal(l0, l1)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    # sampled (batch, query head) pairs, every row, against the checker
+    G = Hq // Hkv
+    sample = sorted({(0, 0), (1, Hq - 1), (2, G), (3, 1), (B // 2, Hq // 2), (B - 1, Hq - 1), (B - 2, 0)})
+    for b, h in sample:
+        hk = h // G
+        wo, wl = oracle.attn_fwd_f64_ex(bits(q[b:b + 1, h:h + 1]), bits(k[b:b + 1, hk:hk + 1]), bits(v[b:b + 1, hk:hk + 1]),
+                                        causal, sc, kv_lens=None if lens is None else lens[b:b + 1],
+                                        key_mask=None if km is None else km[b:b + 1].numpy())
+        assert max_abs(o1[b, h].cpu().float(), wo[0, 0]) <= TOL, (case, b, h)
+        seen = torch.from_numpy(np.isfinite(wl[0, 0]))
+        if bool(seen.any()):
+            assert max_abs(l1[b, h].cpu()[seen], wl[0, 0][seen.numpy()]) <= TOL, (case, b, h)
+        assert bool(torch.isneginf(l1[b, h].cpu()[~seen]).all()), (case, b, h)     # rows that see no key: LSE = -inf
 
 
 # ------------------------------------------- grouped queries, window, key lengths (prefill)

@@ -100,6 +100,37 @@ def test_flash_attn_bwd_grouped_window_lengths(gpu, B, Hq, Hkv, N, D, mode):
             assert float(dv[b, :, n:].float().abs().max() if n < N else 0.0) == 0.0
 
 
+@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("N,D", [(64, 128), (64, 64), (200, 128), (130, 64)])
+def test_flash_attn_bwd_single_visible_key(gpu, N, D, window):
+    # Key length 1: every query row sees key 0 only, so P[i,0] = 1, O[i] = V[0], dS = 0 and
+    #   dV[0] = sum_i dO[i]   (N terms of size ~1: entries of size ~sqrt(N), up to 20-30 at N = 64),   dQ = dK = 0.
+    # A bf16 result of size 16..32 is at best 0.0625 (half a unit in the last place) from the exact sum, which an absolute
+    # tolerance of 3e-2 alone would flag: the rule of this file (3e-2 + 3e-2 |want|, relative Frobenius 1e-2) is the right
+    # one, and the closed form pins the values on top of it: each dV[0] entry within one bf16 rounding of the exact sum.
+    B, Hq, Hkv = 2, 2, 1
+    q, g = lt.make_inputs(8300 + N + D, (B, Hq, N, D), (B, Hq, N, D))
+    k, v = lt.make_inputs(8301 + N + D, (B, Hkv, N, D), (B, Hkv, N, D))
+    sc = 1 / math.sqrt(D)
+    lens = [1, 1]
+    lens_d = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    qd, kd, vd, gd = (t.cuda() for t in (q, k, v, g))
+    o, lse = gpu.flash_attn_fwd(qd, kd, vd, causal=True, scale=sc, window=window, kv_lens=lens_d)
+    assert torch.equal(o, vd[:, :, :1].repeat_interleave(Hq // Hkv, 1).expand(B, Hq, N, D))
+    dq, dk, dv = gpu.flash_attn_bwd(qd, kd, vd, o, lse, gd, causal=True, scale=sc, window=window, kv_lens=lens_d)
+    wq, wk, wv = oracle.attn_bwd_f64_ex(bits(q), bits(k), bits(v), bits(g), True, sc, window=window, kv_lens=lens)
+    check(dq, wq, "dq")
+    check(dk, wk, "dk")
+    check(dv, wv, "dv")
+    exact = g.double().sum(dim=(1, 2))                                   # [B, D]: sum over both query heads and all rows
+    got = dv[:, 0, 0].cpu().double()
+    ulp = torch.exp2(torch.floor(torch.log2(exact.abs().clamp_min(1e-30))) - 7)      # bf16: 8 significant bits
+    assert bool(((got - exact).abs() <= 0.5 * ulp + 1e-4 * math.sqrt(N)).all()), float((got - exact).abs().max())
+    assert float(dv[:, :, 1:].float().abs().max()) == 0.0
+    assert float(dk[:, :, 1:].float().abs().max()) == 0.0
+    assert float(dq.float().abs().max()) <= 1e-3 and float(dk.float().abs().max()) <= 1e-3
+
+
 def test_flash_attn_bwd_properties(gpu):
     # exact linearity in a power-of-two multiple of dO; bit-identical repeat runs (no atomics);
     # rows of dS sum to zero, hence sum_j dK[j] = scale * sum_i (sum_j dS[i,j]) Q[i] = 0.

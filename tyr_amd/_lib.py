@@ -14,7 +14,7 @@ SYMBOLS = (
     "tyr_hip_flash_attn_fwd", "tyr_hip_flash_attn_fwd_gqa", "tyr_hip_flash_attn_bwd_workspace_bytes", "tyr_hip_flash_attn_bwd",
     "tyr_hip_flash_attn_bwd_gqa", "tyr_hip_flash_attn_fwd_mask", "tyr_hip_flash_attn_bwd_mask",
     "tyr_hip_gqa_decode_workspace_bytes", "tyr_hip_gqa_decode_auto_splits",
-    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_bf16_batched", "tyr_hip_gemm_force_general", "tyr_hip_gemm_fp8", "tyr_hip_gemm_fp8_ex",
+    "tyr_hip_gqa_decode", "tyr_hip_gqa_decode_varlen", "tyr_hip_gqa_decode_static", "tyr_hip_gemm_bf16", "tyr_hip_gemm_bf16_batched", "tyr_hip_gemm_force_general", "tyr_hip_flash_attn_fwd_persistent", "tyr_hip_gemm_fp8", "tyr_hip_gemm_fp8_ex",
     "tyr_hip_decode_rope_append", "tyr_hip_rope_fwd", "tyr_hip_layernorm_residual", "tyr_hip_copy", "tyr_hip_mfma_sustain", "tyr_hip_mse_loss_grad_workspace_bytes", "tyr_hip_mse_loss_grad", "tyr_hip_sgd_step",
 )
 
@@ -71,6 +71,8 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_gemm_bf16_batched.restype = ci
     L.tyr_hip_gemm_force_general.argtypes = [ci]
     L.tyr_hip_gemm_force_general.restype = ci
+    L.tyr_hip_flash_attn_fwd_persistent.argtypes = [ci]
+    L.tyr_hip_flash_attn_fwd_persistent.restype = ci
     L.tyr_hip_gemm_fp8.argtypes = [vp, vp, vp, u64, u64, u64, f32, f32, ci, vp]
     L.tyr_hip_gemm_fp8.restype = ci
     L.tyr_hip_gemm_fp8_ex.argtypes = [vp, vp, vp, u64, u64, u64, f32, vp, vp, ci, ci, vp]
@@ -83,7 +85,7 @@ def load() -> ctypes.CDLL:
     L.tyr_hip_layernorm_residual.restype = ci
     L.tyr_hip_copy.argtypes = [vp, vp, sz, vp]
     L.tyr_hip_copy.restype = ci
-    L.tyr_hip_mfma_sustain.argtypes = [vp, sz, ci, u64, u64, vp, ctypes.POINTER(ctypes.c_double), vp]
+    L.tyr_hip_mfma_sustain.argtypes = [vp, sz, ci, u64, u64, vp, sz, ctypes.POINTER(ctypes.c_double), vp]
     L.tyr_hip_mfma_sustain.restype = ci
     L.tyr_hip_mse_loss_grad_workspace_bytes.argtypes = [u64]
     L.tyr_hip_mse_loss_grad_workspace_bytes.restype = sz

@@ -83,9 +83,10 @@ __global__ __launch_bounds__(256) void mfma_sustain_kernel(const unsigned char* 
 }  // namespace tyr
 
 extern "C" int tyr_hip_mfma_sustain(const void* operands, size_t operand_bytes, int dtype, uint64_t workgroups,
-                                    uint64_t iters, float* sink, double* flop_per_launch, void* stream) {
+                                    uint64_t iters, float* sink, size_t sink_bytes, double* flop_per_launch, void* stream) {
     using namespace tyr;
     if (!operands || !sink) return TYR_HIP_ERR_NULL_POINTER;
+    if (workgroups <= (1u << 24) && sink_bytes < (size_t)workgroups * 256 * sizeof(float)) return TYR_HIP_ERR_WORKSPACE;
     if (dtype != TYR_HIP_MFMA_BF16 && dtype != TYR_HIP_MFMA_E4M3) return TYR_HIP_ERR_UNSUPPORTED;
     const size_t span = (size_t)2 * NF * 64 * (dtype == TYR_HIP_MFMA_BF16 ? 16 : 32);
     if (workgroups == 0 || iters == 0 || workgroups > (1u << 24) || iters > (1u << 30) || operand_bytes < span)

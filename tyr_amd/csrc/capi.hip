@@ -57,6 +57,22 @@ int set_gemm_general_only(int on) {
     g_gemm_general.store(on ? 1 : 0);
     return prev;
 }
+static std::atomic<int> g_fa_persistent{-1};         // -1 = not initialised
+bool flash_attn_fwd_persistent() {
+    int v = g_fa_persistent.load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char* e = getenv("TYR_HIP_FA_PERSISTENT");
+        v = (e != nullptr && e[0] == '1') ? 1 : 0;
+        int expected = -1;
+        if (!g_fa_persistent.compare_exchange_strong(expected, v)) v = expected;
+    }
+    return v != 0;
+}
+int set_flash_attn_fwd_persistent(int on) {
+    const int prev = flash_attn_fwd_persistent() ? 1 : 0;
+    g_fa_persistent.store(on ? 1 : 0);
+    return prev;
+}
 }  // namespace tyr
 
 // ---- the entry point that allocates nothing ---------------------------------------------------
@@ -391,6 +407,8 @@ int tyr_hip_gemm_bf16_batched(const void* a, const void* b, void* c, uint64_t ba
 }
 
 int tyr_hip_gemm_force_general(int on) { return tyr::set_gemm_general_only(on); }
+
+int tyr_hip_flash_attn_fwd_persistent(int on) { return tyr::set_flash_attn_fwd_persistent(on); }
 
 int tyr_hip_gemm_fp8(const void* aq, const void* bq, void* c, uint64_t M, uint64_t N, uint64_t K,
                      float scale_a, float scale_b, int trans_b, void* stream) {

@@ -32,12 +32,15 @@
 // pointing at 4 consecutive d of 4 kv rows hand every lane "its" d for those 4 rows.
 #include <limits.h>
 
+#include <atomic>
+
 #include "common.hpp"
 #include "launch.hpp"
 
 namespace tyr {
 
 namespace fa {
+constexpr int kMaxDevices = 64;
 constexpr int BM = 128, BN = 64, THREADS = 256;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
@@ -88,10 +91,11 @@ __global__ __launch_bounds__(fa::THREADS, 2) void flash_attn_fwd_kernel(
     // query heads times ntq tiles share one K/V; the G heads of a tile are adjacent.
     // With `pair` (causal) a workgroup handles query tile ntq-1-tr and then tile tr: every
     // workgroup does the same amount of work and there are half as many of them to start.
-    // A workgroup is persistent: the launch has at most two workgroups per CU, and workgroup p walks the job ids
-    // p, p + gridDim.x, ... (gridDim.x is a multiple of 8, so all of them belong to its XCD).  The hand-over from a
-    // job's last tile to the next job's first one is the hand-over between the two tiles of a pair: no dispatch gap,
-    // and the next tile's K(0), K(1) and Q are requested under the end of the current one.
+    // A launch has either one workgroup per job id, or (persistent launch) two workgroups per CU, of which workgroup p
+    // walks the job ids p, p + gridDim.x, ... (the host makes gridDim.x a multiple of 8 then, so with the XCD mapping
+    // above all of them belong to its XCD).  The hand-over from a job's last tile to the next job's first one is the
+    // hand-over between the two tiles of a pair: the next tile's K(0), K(1) and Q are requested under the end of the
+    // current one.
     const int ntr = pair ? (ntq + 1) / 2 : ntq;  // tile ranks per head
     auto decode = [&](int id, int& bh_, int& tr_, int& kvbh_) {
         const int ngroups = BH / G;              // B * Hkv
@@ -450,14 +454,24 @@ int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, 
     const bool ext = window > 0 || kv_lens != nullptr || key_mask != nullptr;
     const int pair = (causal && window <= 0 && ntq > 1) ? 1 : 0;   // lengths and key masks keep tile 0 starting at key 0
     const int total_ids = BH * (pair ? (ntq + 1) / 2 : ntq);
-    // two workgroups fit a CU (registers, and 64 KB of LDS each at D = 128): that many persistent workgroups
-    static const int resident = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-        return 2 * cus / 8 * 8;
-    }();
-    dim3 grid((unsigned)(total_ids < resident ? total_ids : resident)), block(THREADS);
+    // One workgroup per job id, or persistent workgroups: two per CU (what registers and 64 KB of LDS at D = 128 allow),
+    // rounded down to a multiple of 8 so that a workgroup's job ids stay on one XCD, and never fewer than 8.
+    unsigned nwg = (unsigned)total_ids;
+    if (flash_attn_fwd_persistent()) {
+        static std::atomic<int> resident_of[kMaxDevices];       // per device, 0 = not asked yet
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+        int resident = resident_of[dev].load(std::memory_order_relaxed);
+        if (resident == 0) {
+            int cus = 0;
+            if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+            resident = 2 * cus / 8 * 8;
+            if (resident < 8) resident = 8;
+            resident_of[dev].store(resident, std::memory_order_relaxed);
+        }
+        if (total_ids > resident) nwg = (unsigned)resident;
+    }
+    dim3 grid(nwg), block(THREADS);
     const float scale_log2 = scale * LOG2E;
     auto Qp = static_cast<const uint16_t*>(q);
     auto Kp = static_cast<const uint16_t*>(k);

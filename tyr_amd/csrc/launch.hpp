@@ -18,6 +18,10 @@ int set_gemm_general_only(int on);   // returns the previous value
 // row_scale [M] / col_scale [N] (device f32, may be null); out_kind 0 = bf16, 1 = f32, 2 = e4m3
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
                     int trans_b, const float* row_scale, const float* col_scale, int out_kind, hipStream_t stream);
+// Process-wide choice between persistent forward workgroups (two per CU walking the job ids) and one workgroup per job
+// id.  Its initial value is taken once from the environment variable TYR_HIP_FA_PERSISTENT ("1" = persistent).
+bool flash_attn_fwd_persistent();
+int set_flash_attn_fwd_persistent(int on);   // returns the previous value
 int launch_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
                           int Hq, int Hkv, int N, int D, int causal, int window, const int* kv_lens,
                           const uint8_t* key_mask, float scale, hipStream_t stream);

@@ -74,9 +74,10 @@ __global__ __launch_bounds__(1024) void mse_loss_kernel(const float* __restrict_
     }
 }
 
-// param' = param - (f32(grad) * lr); optionally also bf16(param')
-__global__ __launch_bounds__(THREADS) void sgd_kernel(const float* __restrict__ param, const uint16_t* __restrict__ grad, float lr,
-                                                      float* __restrict__ param_out, uint16_t* __restrict__ param_out_bf16,
+// param' = param - (f32(grad) * lr); optionally also bf16(param').  param_out may be param itself (the in-place update), so
+// neither of the two is declared restrict; a lane stores only the elements it loaded.
+__global__ __launch_bounds__(THREADS) void sgd_kernel(const float* param, const uint16_t* __restrict__ grad, float lr,
+                                                      float* param_out, uint16_t* __restrict__ param_out_bf16,
                                                       size_t pieces) {
     const size_t i = (size_t)blockIdx.x * THREADS + threadIdx.x;
     if (i >= pieces) return;
