@@ -846,11 +846,47 @@ def wl_dsl_h100_gemm(torch, tyr, steps, warmup, cpu, parity):
     return res
 
 
+def wl_dsl_lcf_attn(torch, tyr, steps, warmup, cpu, parity):
+    """The reference's load-compute-finish attention surface for D = 128 (Tyr/GPU/Kernels/MhaH100LCF.lean:29-82,109-132: one
+    64-row query tile per block, 24 KV tiles of 128 rows, i.e. sequence length 3072, non-causal, scale 1/sqrt(128)) emitted
+    for gfx950: a group of two waves per query tile, K and V read from LDS by the products.  The program addresses one
+    [3072, 128] head at column block blockIdx.x, so the heads are laid side by side ([sequence, heads * 128]) and the grid
+    is (heads, 3072 / 64)."""
+    from tyr_amd.dsl import kernels, runtime
+    H, S, D = 64, 3072, 128
+    torch.manual_seed(0)
+    q, k, v = (_normal(torch, S, H * D).to(torch.bfloat16) for _ in range(3))
+    o = torch.zeros(S, H * D, dtype=torch.bfloat16, device="cuda")
+    kern = kernels.tkMhaH100LCFFwd128()
+    fn = lambda: runtime.launch(kern, [q, k, v, o, S, D], grid=(H, S // 64, 1), block=(64, 1, 1))   # 2 warps of the reference
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    tf = 4.0 * H * S * S * D / (ms * 1e-3) / 1e12
+    res = {"metric": "emitted attention TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
+           "dtype": "bf16",
+           "config": {"workload": "tile-DSL program tkMhaH100LCFFwd128 emitted for gfx950: non-causal attention forward, bf16, "
+                                  "64 heads side by side, N=3072 (24 KV tiles of 128), D=128, 64 query rows per two-wave group",
+                      "flop_convention": "4*H*N^2*D (non-causal)"},
+           "roofline": _mfma_roofline(torch, "mfma_bf16", "tkMhaH100LCFFwd128 (emitted)", tf, TRAFFIC.get("dsl_lcf_attn"))}
+    if parity:
+        import numpy as np
+        import oracle
+        e_o = 0.0
+        heads = (0, H - 1)
+        for h in heads:
+            sl = lambda t: _bits(t[:, h * D:(h + 1) * D].contiguous().view(1, 1, S, D))
+            o64, _ = oracle.attn_fwd_f64(sl(q), sl(k), sl(v), False, 0.08838834764)
+            e_o = max(e_o, float(np.abs(o[:, h * D:(h + 1) * D].cpu().float().numpy() - o64[0, 0]).max()))
+        res["parity"] = _parity(tol=2e-2, max_abs_o=e_o,
+                                sample=f"heads {list(heads)}, all 3072 rows, against the float64 checker (oracle.attn_fwd_f64)")
+    return res
+
+
 WORKLOADS = {"attn_fwd_causal": wl_attn, "attn_bwd_causal": wl_attn_bwd, "mha_train_step": wl_train_step,
              "mha_train_step_ref_shape": wl_train_step_ref_shape, "gqa_decode": wl_decode, "gqa_decode_split4": wl_decode_split4,
              "gqa_decode_small_batch": wl_decode_small_batch, "gemm_bf16": wl_gemm_bf16,
              "gemm_fp8": wl_gemm_fp8, "decode_step": wl_decode_step, "rope_fwd": wl_rope, "layernorm_residual": wl_layernorm,
-             "copy_kernel": wl_copy_kernel, "dsl_simple_gemm": wl_dsl_simple_gemm, "dsl_h100_gemm": wl_dsl_h100_gemm}
+             "copy_kernel": wl_copy_kernel, "dsl_simple_gemm": wl_dsl_simple_gemm, "dsl_h100_gemm": wl_dsl_h100_gemm,
+             "dsl_lcf_attn": wl_dsl_lcf_attn}
 CALIBRATION = {"copy_1gib": wl_copy, "mfma_sustain_bf16": wl_mfma_bf16, "mfma_sustain_fp8": wl_mfma_fp8}
 
 

@@ -215,7 +215,8 @@ def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None, str
     any statement that overwrites a shared object read since the last barrier, loop back-edges
     included.  (Read-after-write needs nothing: all waves write identical data and a wave reads
     after its own write.)  A conditional body cannot hold a barrier, so the barrier goes in front of
-    the conditional."""
+    the conditional.  Where only what was read *before* a loop is overwritten inside it, one barrier goes
+    in front of the loop instead of one into every iteration."""
     shared = {s.v for s in walk(kernel.body) if s.op in ("declST", "declSV")}
     regions = regions or {}
 
@@ -250,33 +251,46 @@ def shared_hazard_barriers(kernel: Kernel, regions: Dict[VarId, Any] = None, str
             w |= b
         return r, w
 
-    marks = set()
-
-    def run(body, pending: set, mark: bool) -> set:
+    def run(body, pending: set, marks) -> set:
+        """Walks a statement list; `marks` (a set, or None for a dry run) collects the statements that need a barrier."""
         for s in body:
             if s.op == "sync":
                 pending = set()
             elif s.op in ("forLoop", "forLoopVal"):
-                end = run(s.body, set(pending), False)
-                end = run(s.body, pending | end, mark)               # second pass sees the back-edge
-                pending = pending | end
+                # hazards of the loop by itself (entry state = what its own back edge brings) ...
+                own = set()
+                run(s.body, run(s.body, set(), None), own)
+                # ... and with what is pending from before the loop
+                full = set()
+                end = run(s.body, pending | run(s.body, set(pending), None), full)   # second pass sees the back-edge
+                if full != own:
+                    # reads from before the loop are overwritten inside it: one barrier in front of the loop
+                    if marks is not None:
+                        marks.add(id(s))
+                        marks |= own
+                    pending = run(s.body, run(s.body, set(), None), None)
+                else:
+                    if marks is not None:
+                        marks |= full
+                    pending = pending | end
             elif s.op == "ifStmt":
                 r, w = all_rw(s.thenBody + s.elseBody)
                 if w & pending:
-                    if mark:
+                    if marks is not None:
                         marks.add(id(s))
                     pending = set()
                 pending = pending | r
             else:
                 r, w = rw(s)
                 if w & pending:
-                    if mark:
+                    if marks is not None:
                         marks.add(id(s))
                     pending = set()
                 pending = pending | r
         return pending
 
-    run(kernel.body, set(), True)
+    marks = set()
+    run(kernel.body, set(), marks)
     return marks
 
 
@@ -423,9 +437,10 @@ def row_split_set(kernel: Kernel, rv_layout: Dict[VarId, str], streamed: Dict[Va
     return split
 
 
-def peak_tile_registers(kernel: Kernel, split=frozenset(), waves: int = 1, streamed=frozenset()) -> int:
+def peak_tile_registers(kernel: Kernel, split=frozenset(), waves: int = 1, streamed=frozenset(), packed: bool = False) -> int:
     """Most registers per lane the register tiles live at one point need (a tile lives from its first to its
-    last mention; a mention inside a loop counts for the whole loop)."""
+    last mention; a mention inside a loop counts for the whole loop).  One register per element, or -- `packed` --
+    what the elements' bytes really take (two bf16 or four fp8 values per register)."""
     decl = {s.v: s for s in walk(kernel.body) if s.op == "declRT"}
     live: Dict[VarId, List[int]] = {}
     pos = [0]
@@ -451,7 +466,8 @@ def peak_tile_registers(kernel: Kernel, split=frozenset(), waves: int = 1, strea
     run(kernel.body)
     peak = 0
     for p_ in range(1, pos[0] + 1):
-        need = sum(_rt_regs(decl[v], decl[v].rows // waves if v in split else None) for v, r in live.items() if r[0] <= p_ <= r[1])
+        need = sum(_rt_regs(decl[v], decl[v].rows // waves if v in split else None) *
+                   (_DTYPE_BYTES.get(decl[v].dtype, 4) if packed else 4) // 4 for v, r in live.items() if r[0] <= p_ <= r[1])
         peak = max(peak, need)
     return peak
 
@@ -491,17 +507,41 @@ class _Emitter:
         # request the next iteration's global tiles of a loop before the work of the current one
         self.prefetch_global_loads = prefetch_global_loads
         # LDS tiles with disjoint live ranges share storage
-        # (only where that asks for no barrier the program does not already have)
+        # (only where that puts no additional barrier into a loop)
         self.lds = lds_plan(kernel) if share_lds else {}
-        if self.lds and shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds), self.streamed) != \
-                shared_hazard_barriers(kernel, None, self.streamed):
-            self.lds = {}
+        if self.lds:
+            in_loops = {id(t) for l in walk(kernel.body) if l.op in ("forLoop", "forLoopVal") for t in walk(l.body)}
+            extra = shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds), self.streamed) - \
+                shared_hazard_barriers(kernel, None, self.streamed)
+            if extra & in_loops:
+                self.lds = {}
         self.barrier_before = shared_hazard_barriers(kernel, _lds_regions(kernel, self.lds), self.streamed) \
             if hazard_barriers else set()
         # waves per workgroup the kernel is compiled for; 4 (one per SIMD) leaves every wave the
         # full 512-register file, and covers the 128-thread blocks the reference's runners launch.
         # A wave group needs exactly its own number of waves.
         self.max_waves = self.waves if self.group else max_waves
+        self.min_blocks = self._blocks_per_cu()
+
+    def _blocks_per_cu(self) -> int:
+        """Workgroups per CU the kernel is compiled for.  A wave-group program runs with exactly its own number of waves, so
+        when two such workgroups fit a CU -- LDS, and 256 registers per lane at two waves per SIMD -- the compiler is told to
+        keep to that budget: a second resident workgroup hides the first one's global latency and its epilogue."""
+        if not self.group:
+            return 1
+        decl = {t.v: t for t in walk(self.k.body) if t.op == "declST"}
+        size = {v: (d.rows * (d.cols * _DTYPE_BYTES.get(d.dtype, 4) + 16) + 15) // 16 * 16 for v, d in decl.items()}
+        lds = max((off + size[v] for v, off in self.lds.items()), default=0) if self.lds else sum(size.values())
+        if 2 * lds > 160 * 1024:
+            return 1
+        if 2 * self.waves <= 4:
+            return 2                                     # still one wave per SIMD: the whole register file each
+        regs = peak_tile_registers(self.k, self.split, self.waves, set(self.streamed), packed=True)
+        for l in (t for t in walk(self.k.body) if t.op in ("forLoop", "forLoopVal")):
+            if self.prefetch_global_loads:
+                regs += sum(self.info[t.dst].rows * self.info[t.dst].cols * _DTYPE_BYTES[self.info[t.dst].dtype] // (256 * self.waves)
+                            for t in self.prefetchable(l))
+        return 2 if regs <= 248 else 1               # the rest of the 256 goes to addresses and operand fragments
 
     def kind(self, v: VarId) -> str:
         s = self.info.get(v)
@@ -707,8 +747,8 @@ class _Emitter:
                     defined.add(x)
         out = []
         for t in loop.body:
-            if t.op == "comment":
-                continue
+            if t.op == "comment" or self._registers_only(t):
+                continue                                 # declarations and register work in front of the loads stay where they are
             if t.op != "loadGlobal" or id(t) in self.barrier_before:
                 break
             free = all(c == loop.v or c not in defined for c in (t.coordB, t.coordD, t.coordR, t.coordC))
@@ -725,6 +765,16 @@ class _Emitter:
             if not all(even(t) for t in out):
                 return []
         return out
+
+    def _registers_only(self, t: Stmt) -> bool:
+        """A statement that touches register tiles / vectors and compile-time values only (no LDS, no global memory,
+        no control flow)."""
+        if t.op in ("forLoop", "forLoopVal", "ifStmt", "sync", "raw", "transpose", "swapLayout") or t.op in NVIDIA_ONLY:
+            return False
+        if t.op not in ("declRT", "declRV", "unary", "binary", "ternary", "scalarMul", "scalarAdd", "convert", "broadcast",
+                        "binaryBroadcast", "vecFillScalar", "vecIota", "constInt", "constFloat"):
+            return False
+        return all(self.kind(a) in ("RT", "RV", "scalar") for a in t.args if isinstance(a, VarId))
 
     def prefetched_loop(self, loop: Stmt, hi: str, pre, ind: str) -> str:
         I = lambda v: v.ident
@@ -870,7 +920,8 @@ class _Emitter:
             head = (f"  // run by a group of {self.waves} waves: row-tied register tiles are cut into {self.waves} row slices\n"
                     f"  const int tyr_wave = wave::index();\n")
         self.dirty = set()
-        return (f"__global__ __launch_bounds__({64 * self.max_waves}) void {self.k.name}({sig}) {{\n" + pool + head +
+        bounds = f"{64 * self.max_waves}, {self.min_blocks}" if self.min_blocks > 1 else f"{64 * self.max_waves}"
+        return (f"__global__ __launch_bounds__({bounds}) void {self.k.name}({sig}) {{\n" + pool + head +
                 self.body(self.k.body, "  ") + "}\n")
 
     def launcher_signature(self) -> str:
