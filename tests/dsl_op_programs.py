@@ -313,7 +313,80 @@ def dslOpsScanAtomic() -> Kernel:
     return k.build()
 
 
-ALL = (dslOpsScanAtomic, dslOpsUnary, dslOpsBinary, dslOpsMasks, dslOpsLayout, dslOpsMma, dslOpsControl)
+FULL_TILE_BLOCKS = ("fmaAxBtC", "fmaAxCtB", "transposeInPlace")
+FULL_VECTOR_BLOCKS = ("fullMaxOfVec", "fullSumOfVec", "fullMinOfTile", "fullSumOfTile", "fullSumAccum", "fullCumsum",
+                      "fullCumprod", "fullSumOfColVec")
+
+
+def dslOpsFull() -> Kernel:
+    """The IR's "Full" axis (reductions over every element, scans along a vector), the two matrix-style FMA tags and the
+    in-place transpose of a square tile.  x, y, z 64x64 f32, v 64 f32.  Tile results go to `out` in the order of
+    FULL_TILE_BLOCKS, vector results to `vout` in the order of FULL_VECTOR_BLOCKS (a full reduction leaves its result in
+    every element of its destination)."""
+    from tyr_amd.dsl.ir import stmt
+    from tyr_amd.dsl.builder import RTileCoord
+    k = KernelBuilder("dslOpsFull")
+    x_ptr = k.gptr("Float32", "x")
+    y_ptr = k.gptr("Float32", "y")
+    z_ptr = k.gptr("Float32", "z")
+    v_ptr = k.gptr("Float32", "v")
+    out = k.gptr("Float32", "out")
+    vout = k.gptr("Float32", "vout")
+    coord = k.blockCoord2D()
+    xs, ys, zs = (k.allocST("Float32", T, T) for _ in range(3))
+    stage = k.allocST("Float32", T, T)
+    vs = k.allocSV("Float32", T)
+    x, y, z, w = (k.allocRT("Float32", T, T) for _ in range(4))
+    k.loadGlobal(xs, x_ptr, coord)
+    k.loadGlobal(ys, y_ptr, coord)
+    k.loadGlobal(zs, z_ptr, coord)
+    k.loadVecGlobalRow(vs, v_ptr, coord)
+    k.sync()
+    k.load(x, xs)
+    k.load(y, ys)
+    k.load(z, zs)
+    k.emit(stmt("ternary", "FMAAxBtC", w.id, x.id, y.id, z.id))        # x * y + z
+    _emit_tile(k, out, stage, w, 0)
+    k.emit(stmt("ternary", "FMAAxCtB", w.id, x.id, y.id, z.id))        # x * z + y
+    _emit_tile(k, out, stage, w, 1)
+    k.copy(w, x)
+    k.transpose(w, w)
+    _emit_tile(k, out, stage, w, 2)
+
+    z0 = k.constIntVal(0)
+
+    def put(vec, i):
+        k.sync()
+        k.storeVec(vs, vec)
+        k.storeVecGlobal(vout, vs, RTileCoord(z0, z0, z0, k.constIntVal(i)))
+
+    v = k.allocRV("Float32", T)
+    k.loadVec(v, vs)
+    r = k.allocRV("Float32", T)
+    k.emit(stmt("reduce", "Max", "Full", r.id, v.id))
+    put(r, 0)
+    k.emit(stmt("reduce", "Sum", "Full", r.id, v.id))
+    put(r, 1)
+    k.emit(stmt("reduce", "Min", "Full", r.id, x.id))
+    put(r, 2)
+    k.emit(stmt("reduce", "Sum", "Full", r.id, x.id))
+    put(r, 3)
+    acc = k.allocRV("Float32", T)
+    k.copyVec(acc, v)
+    k.emit(stmt("reduceAccum", "Sum", "Full", r.id, v.id, acc.id))     # sum(v) + v[i]
+    put(r, 4)
+    k.emit(stmt("cumsum", "Full", r.id, v.id))
+    put(r, 5)
+    k.emit(stmt("cumprod", "Full", r.id, v.id))
+    put(r, 6)
+    c = k.allocRV("Float32", T)
+    k.colSum(c, x)                                                     # a per-column vector (the other register layout)
+    k.emit(stmt("reduce", "Sum", "Full", r.id, c.id))
+    put(r, 7)
+    return k.build()
+
+
+ALL = (dslOpsScanAtomic, dslOpsUnary, dslOpsBinary, dslOpsMasks, dslOpsLayout, dslOpsMma, dslOpsControl, dslOpsFull)
 
 
 # ---- build step (run by __graft_entry__.build(); the tests only load what it built)

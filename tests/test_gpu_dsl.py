@@ -206,9 +206,12 @@ def test_mha_h100_lcf_forward_programs(rt, name, D):
     want = p @ v[0, 0].double()
     assert max_abs(o[0, 0].cpu().float(), want) <= 2e-2
     assert float((o[0, 0].cpu().double() - want).norm() / want.norm()) <= 1e-2
-    # any other block size is refused: the compiled program is a group of exactly two waves
-    with pytest.raises(RuntimeError, match="invalid launch arguments"):
-        runtime.launch(getattr(kernels, name)(), [q.cuda(), k.cuda(), v.cuda(), o, nkv, D], grid=(1, 1, 1), block=(128, 1, 1))
+    # the compiled program is a group of exactly two waves: the launcher starts two, whatever block shape it is given
+    # (every warp of the reference's block repeats the whole tile program, so the result does not depend on it)
+    o2 = torch.zeros_like(o)
+    runtime.launch(getattr(kernels, name)(), [q.cuda(), k.cuda(), v.cuda(), o2, nkv, D], grid=(1, nq // 64, 1), block=(128, 1, 1))
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2)
 
 
 @pytest.mark.parametrize("M,N", [(128, 256), (384, 1024)])
@@ -271,3 +274,104 @@ def test_tkH100Fp8ScaledGemmFwd(rt):
     want = torch.from_numpy(want_f32) * sa[:, None] * sb[None, :]
     rel = float((c.cpu() - want).norm() / want.norm())
     assert rel <= 1e-4, rel                                   # f32 accumulation order is the only difference
+
+
+# ------------------------------------------------------------------ the reference's demonstration programs with makeCausal
+def _causal_demo_reference(q, k, v, explicit_softmax):
+    """What `flashAttnFwdNew` / `flashAttnFwdWithLse` (FlashAttn.lean:26-95, FlashAttnBwd.lean:25-103) and `flashAttnFwd`
+    (Examples.lean:93-144) compute for one 64-row query tile, statement by statement in float64 on the bf16 inputs: no score
+    scale, the causal mask inside every 64 x 64 tile (fill -1e10), and a score tile that is never cleared -- the scores of KV
+    block j start from the probabilities of block j-1 (zeros for block 0, the value-initialised tile).  P is rounded to bf16
+    before P V, as `convert p s` does."""
+    q, k, v = q.double(), k.double(), v.double()
+    s = torch.zeros(64, 64, dtype=torch.float64)
+    o = torch.zeros(64, 64, dtype=torch.float64)
+    row_max = torch.full((64,), -float("inf"), dtype=torch.float64)
+    row_sum = torch.zeros(64, dtype=torch.float64)
+    keep = torch.ones(64, 64, dtype=torch.bool).tril()
+    for j in range(4):
+        s = q @ k[64 * j:64 * j + 64].T + s
+        s = torch.where(keep, s, torch.full_like(s, -1e10))
+        prev = row_max
+        row_max = torch.maximum(row_max, s.max(dim=1).values)
+        if not explicit_softmax:                              # onlineSoftmax rescales what it has accumulated
+            scale = torch.exp(prev - row_max)
+            o = o * scale[:, None]
+            row_sum = row_sum * scale
+        s = torch.exp(s - row_max[:, None])
+        row_sum = row_sum + s.sum(dim=1)
+        o = o + s.bfloat16().double() @ v[64 * j:64 * j + 64]
+    return o / row_sum[:, None], torch.log(row_sum) + row_max
+
+
+@pytest.mark.parametrize("name", ["flashAttnFwdNew", "flashAttnFwdWithLse", "flashAttnFwd"])
+def test_causal_demonstration_forwards(rt, name):
+    kernels, runtime = rt
+    # small scores (inputs of std 0.3), as unscaled 64-term dot products of N(0,1) values would saturate the softmax
+    q, k, v = lt.make_inputs(71, (128, 64), (256, 64), (256, 64), std=0.3)
+    o = torch.zeros(128, 64, dtype=torch.bfloat16).cuda()
+    lse = torch.zeros(128).cuda()
+    args = [q.cuda(), k.cuda(), v.cuda(), o] + ([lse] if name == "flashAttnFwdWithLse" else []) + [256, 64]
+    runtime.launch(getattr(kernels, name)(), args, grid=(1, 2, 1), block=(32, 1, 1))
+    torch.cuda.synchronize()
+    for t in range(2):                                        # query tile t (the KV tiles are the same four for both)
+        want_o, want_lse = _causal_demo_reference(q[64 * t:64 * t + 64], k, v, explicit_softmax=(name == "flashAttnFwd"))
+        got = o[64 * t:64 * t + 64].cpu().float()
+        assert torch.allclose(got, want_o.float(), rtol=3e-2, atol=3e-2), (name, t)
+        assert max_abs(got, want_o) <= 2e-2, (name, t)
+        if name == "flashAttnFwdWithLse":
+            assert max_abs(lse[64 * t:64 * t + 64].cpu(), want_lse) <= 2e-2, (name, t)
+
+
+def test_simpleGemmNew(rt):
+    kernels, runtime = rt
+    M, N, K = 128, 192, 512
+    a, b = lt.make_inputs(4, (M, K), (K, N), std=K ** -0.25)
+    c = torch.zeros(M, N).cuda()
+    runtime.launch(kernels.simpleGemmNew(), [a.cuda(), b.cuda(), c, M, N, K], grid=(N // 64, M // 64, 1), block=(32, 1, 1))
+    torch.cuda.synchronize()
+    want = a.double() @ b.double()
+    assert float((c.cpu().double() - want).norm() / want.norm()) <= 1e-5
+
+
+def test_tkH100Fp8E4M3GemmFwd(rt):
+    """PrecisionGemm.lean:73-89: E4M3 x E4M3 -> f32 -> E4M3.  Inputs are scaled so that the results lie inside the E4M3
+    range; every output must be the E4M3 rounding of its f32 sum (ties and the pipe's accumulation order leave a code of
+    slack on a few elements)."""
+    kernels, runtime = rt
+    M, N, K = 128, 512, 512
+    torch.manual_seed(34)
+    aq = (torch.randn(M, K) * 0.5).to(torch.float8_e4m3fn)
+    bq = (torch.randn(N, K) * 0.5).to(torch.float8_e4m3fn)
+    c = torch.zeros(M, N, dtype=torch.uint8).cuda().view(torch.float8_e4m3fn)
+    runtime.launch(kernels.tkH100Fp8E4M3GemmFwd(), [aq.cuda(), bq.cuda(), c, M, N, K], grid=(N // 256, M // 64, 1),
+                   block=(32, 1, 1))
+    torch.cuda.synchronize()
+    _, want_f32 = oracle.gemm_fp8(aq.view(torch.uint8).numpy(), bq.view(torch.uint8).numpy(), 1.0, 1.0, trans_b=True)
+    wf = torch.from_numpy(want_f32)
+    assert float(wf.abs().max()) < 448.0
+    got = c.cpu().float()
+    want = wf.to(torch.float8_e4m3fn).float()
+    assert float((got != want).float().mean()) <= 0.02
+    assert bool(((got - wf).abs() <= wf.abs() * 2.0 ** -3 + 2.0 ** -9).all())          # never more than one code away
+    rel = float((got - wf).norm() / wf.norm())
+    assert rel <= 4e-2, rel                                   # E4M3 keeps 3 mantissa bits: rounding alone is ~2.5e-2
+
+
+@pytest.mark.parametrize("M,N", [(128, 256), (256, 768)])
+def test_tkB200Fp8E4M3Gemm1CtaFwd(rt, M, N):
+    """PrecisionGemm.lean:117-133: E4M3 x E4M3 -> f32 -> bf16 on 128 x 256 tiles, run by a group of four waves with the
+    E4M3 B tile read from LDS by the products."""
+    kernels, runtime = rt
+    K = 512
+    aq, _, bq, _ = _fp8_inputs(35, M, N, K)
+    c = torch.zeros(M, N, dtype=torch.bfloat16).cuda()
+    runtime.launch(kernels.tkB200Fp8E4M3Gemm1CtaFwd(), [aq.cuda(), bq.cuda(), c, M, N, K], grid=(N // 256, M // 128, 1),
+                   block=(128, 1, 1))
+    torch.cuda.synchronize()
+    want_bits, want_f32 = oracle.gemm_fp8(aq.view(torch.uint8).numpy(), bq.view(torch.uint8).numpy(), 1.0, 1.0, trans_b=True)
+    got, wf = c.cpu().float(), torch.from_numpy(want_f32)
+    rel = float((got - wf).norm() / wf.norm())
+    assert rel <= 1e-2 and rel <= 3e-3, rel
+    assert bool(((got - wf).abs() <= wf.abs() * 2.0 ** -8 * 1.01 + 16.0).all())
+    assert float((got != from_bits(want_bits).float()).float().mean()) <= 0.05

@@ -175,3 +175,27 @@ def test_scans_and_atomic_accumulation(rt, block):
     assert torch.allclose(acc.cpu(), acc0 + waves * x, rtol=1e-6, atol=1e-6)
     rs = x.sum(1)
     assert torch.allclose(vacc.cpu(), vacc0 + waves * torch.cat([rs, rs]), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("block", [32, 128])
+def test_full_axis_fma_tags_and_in_place_transpose(rt, block):
+    P, runtime, L = rt
+    g = torch.Generator().manual_seed(9)
+    x, y, z = (torch.rand(T, T, generator=g) * 0.5 + 0.75 for _ in range(3))
+    v = torch.rand(T, generator=g) * 0.1 + 0.95
+    out = torch.full((len(P.FULL_TILE_BLOCKS) * T, T), 77.0).cuda()
+    vout = torch.full((len(P.FULL_VECTOR_BLOCKS) * T,), 77.0).cuda()
+    runtime.launch(P.dslOpsFull(), [x.cuda(), y.cuda(), z.cuda(), v.cuda(), out, vout], block=(block, 1, 1), library=L)
+    torch.cuda.synchronize()
+    xd, yd, zd, vd = x.double(), y.double(), z.double(), v.double()
+    want_t = {"fmaAxBtC": xd * yd + zd, "fmaAxCtB": xd * zd + yd, "transposeInPlace": xd.T}
+    for i, name in enumerate(P.FULL_TILE_BLOCKS):
+        got = out[i * T:(i + 1) * T].cpu().double()
+        assert torch.allclose(got, want_t[name], rtol=1e-6, atol=1e-6), name
+    ones = torch.ones(T, dtype=torch.float64)
+    want_v = {"fullMaxOfVec": vd.max() * ones, "fullSumOfVec": vd.sum() * ones, "fullMinOfTile": xd.min() * ones,
+              "fullSumOfTile": xd.sum() * ones, "fullSumAccum": vd.sum() + vd, "fullCumsum": vd.cumsum(0),
+              "fullCumprod": vd.cumprod(0), "fullSumOfColVec": xd.sum() * ones}
+    for i, name in enumerate(P.FULL_VECTOR_BLOCKS):
+        got = vout[i * T:(i + 1) * T].cpu().double()
+        assert torch.allclose(got, want_v[name], rtol=2e-5, atol=1e-5), (name, got[:4], want_v[name][:4])

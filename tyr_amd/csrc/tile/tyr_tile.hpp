@@ -707,6 +707,83 @@ __device__ __forceinline__ void outer(rt<T, R, C, layout::row>& dst, const rv<TV
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(a.data[rb][0]) * to_f(b.data[cb][s]));
 }
 
+// ---------------------------------------------------------------- full reductions and scans (vectors, tiles)
+// The reference's IR has a third axis, "Full" (Tyr/GPU/Codegen/AST.lean:54-63; printed as the unprefixed warp::max /
+// warp::sum / warp::cumsum, i.e. the vector forms): the reduction of every element, here left in every element of the
+// destination vector, and the running reduction along a vector.
+namespace detail {
+// OP over the `len` elements of a vector, on every lane.  ALIGN: lane (r, g) holds element 32b + r (both halves the same
+// value); ORTHO: slot s of lane half g holds element 32b + 8(s/4) + 4g + s%4 (every row lane the same value).
+template <typename OP, typename T, int N, vlayout V>
+__device__ __forceinline__ float reduce_all(const rv<T, N, V>& src) {
+    float acc = to_f(src.data[0][0]);
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (V == vlayout::align ? 1 : 16); ++s)
+            if (b != 0 || s != 0) acc = OP::f(acc, to_f(src.data[b][s]));
+    if constexpr (V == vlayout::align) {
+#pragma unroll
+        for (int m = 1; m < 32; m <<= 1) acc = OP::f(acc, lane_xor(acc, m));
+    } else {
+        acc = OP::f(acc, xor32(acc));
+    }
+    return acc;
+}
+}  // namespace detail
+template <typename OP, typename T, int ND, vlayout VD, int N, vlayout V>
+__device__ __forceinline__ void full_reduce(rv<T, ND, VD>& dst, const rv<T, N, V>& src) {
+    const float x = detail::reduce_all<OP>(src);
+#pragma unroll
+    for (int b = 0; b < ND / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (VD == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(x);
+}
+template <typename OP, typename T, int ND, vlayout VD, int N, vlayout V>
+__device__ __forceinline__ void full_reduce(rv<T, ND, VD>& dst, const rv<T, N, V>& src, const rv<T, ND, VD>& accum) {
+    const float x = detail::reduce_all<OP>(src);
+#pragma unroll
+    for (int b = 0; b < ND / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (VD == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(OP::f(x, to_f(accum.data[b][s])));
+}
+// every element of a ROW tile: rows first, then the row results
+template <typename OP, typename T, int ND, vlayout VD, int R, int C>
+__device__ __forceinline__ void full_reduce(rv<T, ND, VD>& dst, const rt<T, R, C, layout::row>& src) {
+    rv<float, R, vlayout::align> rows;
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) {
+        float acc = to_f(src.data[rb][0][0]);
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int s = (cb == 0 ? 1 : 0); s < 16; ++s) acc = OP::f(acc, to_f(src.data[rb][cb][s]));
+        rows.data[rb][0] = OP::f(acc, xor32(acc));
+    }
+    const float x = detail::reduce_all<OP>(rows);
+#pragma unroll
+    for (int b = 0; b < ND / 32; ++b)
+#pragma unroll
+        for (int s = 0; s < (VD == vlayout::align ? 1 : 16); ++s) dst.data[b][s] = from_f<T>(x);
+}
+// dst[i] = OP over i' <= i of src[i'] along an ALIGN vector: a scan over the 32 row lanes, carried from block to block
+template <typename OP, typename T, int N>
+__device__ __forceinline__ void full_scan(rv<T, N, vlayout::align>& dst, const rv<T, N, vlayout::align>& src) {
+    float carry = 0.0f;
+#pragma unroll
+    for (int b = 0; b < N / 32; ++b) {
+        float x = to_f(src.data[b][0]);
+#pragma unroll
+        for (int d = 1; d < 32; d <<= 1) {
+            const float up = __shfl_up(x, d, 32);
+            if (lr() >= d) x = OP::f(up, x);
+        }
+        if (b > 0) x = OP::f(carry, x);
+        dst.data[b][0] = from_f<T>(x);
+        carry = __shfl(x, 31, 32);
+    }
+}
+
 // ---------------------------------------------------------------- scans (ROW tiles)
 // row_scan: dst[i][j] = OP over j' <= j of src[i][j'].  A lane owns the 4-column groups 8q + 4g of
 // its row; group totals are exchanged with the other lane half and prefixed in column order.
@@ -879,6 +956,48 @@ __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const r
                     acc[mb] = mfma_32x32x16_bf16(fb, fa, acc[mb]);
                 }
             }
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+    }
+}
+// E4M3 operands, B as [N, K] rows in LDS: a lane's 32 bytes of k for the 32x32x64 MFMA are the 16 bytes of its slots in two
+// adjacent 32-column blocks (the map of the register tiles), i.e. eight 4-byte pieces at columns 32kb + 8q + 4g.
+template <int M, int N, int K>
+__device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<fp8e4m3, M, K, layout::row>& a,
+                                        const st<fp8e4m3, N, K>& b, const rt<float, M, N, layout::row>& c) {
+    static_assert(K % 64 == 0, "E4M3 products consume k in steps of 64");
+#pragma unroll
+    for (int nb = 0; nb < N / 32; ++nb) {
+        f32x16 acc[M / 32];
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+#pragma unroll
+        for (int kb = 0; kb < K / 32; kb += 2) {
+            i32x8 fb;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int wd = 0; wd < 4; ++wd)
+                    fb[4 * h + wd] = *reinterpret_cast<const int*>(b.at(32 * nb + lr(), 32 * (kb + h) + 8 * wd + 4 * lg()));
+#pragma unroll
+            for (int mb = 0; mb < M / 32; ++mb) {
+                i32x8 fa;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int wd = 0; wd < 4; ++wd) {
+                        uint32_t ua = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) ua |= (uint32_t)a.data[mb][kb + h][4 * wd + e].bits << (8 * e);
+                        fa[4 * h + wd] = (int)ua;
+                    }
+                acc[mb] = mfma_32x32x64_e4m3(fb, fa, acc[mb]);
+            }
+        }
 #pragma unroll
         for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll

@@ -84,7 +84,13 @@ def infer_rv_layouts(kernel: Kernel) -> Dict[VarId, str]:
             parent[find(v)] = find(vs[0])
 
     for s in walk(kernel.body):
-        if s.op == "reduce":
+        if s.op in ("reduce", "reduceAccum") and s.axis == "Full":
+            if s.op == "reduceAccum":                    # any layout serves: the result lands in every element
+                tie(s.dst, s.accum)
+        elif s.op in ("cumsum", "cumprod") and s.axis == "Full":
+            need(s.dst, "align")
+            need(s.src, "align")
+        elif s.op == "reduce":
             need(s.dst, "align" if s.axis == "Row" else "ortho")
         elif s.op == "reduceAccum":
             lay = "align" if s.axis == "Row" else "ortho"
@@ -324,14 +330,15 @@ def streamed_operands(kernel: Kernel) -> Dict[VarId, VarId]:
     cand = {}
     for v, us in uses.items():
         d = info[v]
-        if d.dtype != "BFloat16":
+        if d.dtype not in ("BFloat16", "FP8E4M3"):
             continue
         ok = True
         for u in us:
             if u.op == "load" and u.dst == v and u.src in info and info[u.src].op == "declST":
                 continue
             if u.op == "mma" and u.b == v and v not in (u.dst, u.a, u.c) and (
-                    (u.trans == "ABt" and d.layout == "Row") or (u.trans == "AB" and d.layout == "Col")):
+                    (u.trans == "ABt" and d.layout == "Row") or
+                    (u.trans == "AB" and d.layout == "Col" and d.dtype == "BFloat16")):
                 continue
             ok = False
         if ok and any(u.op == "load" for u in us) and any(u.op == "mma" for u in us):
@@ -561,7 +568,9 @@ class _Emitter:
             if s.v in self.streamed:
                 return f"{ind}// {I(s.v)} stays in LDS: products read their fragments from {I(self.streamed[s.v])}\n"
             rows = s.rows // self.waves if s.v in self.split else s.rows
-            return f"{ind}rt<{_cpp_type(s.dtype)}, {rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)};\n"
+            # (value-initialised: a program that accumulates into a tile it never wrote reads zeros, not whatever the
+            #  registers held; where the tile is written first the compiler drops the zeros)
+            return f"{ind}rt<{_cpp_type(s.dtype)}, {rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)}{{}};\n"
         if op == "declST":
             ty = f"st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}>"
             if s.v in self.lds:
@@ -569,7 +578,7 @@ class _Emitter:
             return f"{ind}__shared__ {ty} {I(s.v)};\n"
         if op == "declRV":
             n = s.len // self.waves if s.v in self.split else s.len
-            return f"{ind}rv<{_cpp_type(s.dtype)}, {n}, vlayout::{self.rv_layout[s.v]}> {I(s.v)};\n"
+            return f"{ind}rv<{_cpp_type(s.dtype)}, {n}, vlayout::{self.rv_layout[s.v]}> {I(s.v)}{{}};\n"
         if op == "declSV":
             return f"{ind}__shared__ sv<{_cpp_type(s.dtype)}, {s.len}> {I(s.v)};\n"
         if op == "declGPtr":
@@ -607,9 +616,11 @@ class _Emitter:
             at = f"coord{{(int){I(s.coordB)}, (int){I(s.coordD)}, (int){I(s.coordR)}, (int){I(s.coordC)}}}"
             return f"{ind}wave::store_add({I(s.dst)}, {I(s.src)}, {at});\n"
         if op in ("cumsum", "cumprod"):
-            if s.axis == "Full":
-                raise UnsupportedStatement("full scans have no gfx950 lowering")
             f = "op_add" if op == "cumsum" else "op_mul"
+            if s.axis == "Full":                         # the vector form: a running reduction along a register vector
+                if self.kind(s.src) != "RV" or self.kind(s.dst) != "RV" or self.rv_layout[s.src] != "align":
+                    raise UnsupportedStatement("a full scan runs along a per-row register vector")
+                return f"{ind}wave::full_scan<{f}>({I(s.dst)}, {I(s.src)});\n"
             return f"{ind}wave::{s.axis.lower()}_scan<{f}>({I(s.dst)}, {I(s.src)});\n"
         if op == "loadScalarGlobal":
             return f"{ind}const auto {I(s.dst)} = {I(s.src)}.ptr[{I(s.offset)}];\n"
@@ -628,9 +639,10 @@ class _Emitter:
         if op == "binary":
             return f"{ind}wave::binary<{BINARY[s.args[0]]}>({I(s.dst)}, {I(s.a)}, {I(s.b)});\n"
         if op == "ternary":
-            if s.args[0] != "FMA":
-                raise UnsupportedStatement(f"ternary {s.args[0]} has no gfx950 lowering")
-            return f"{ind}wave::fma({I(s.dst)}, {I(s.a)}, {I(s.b)}, {I(s.c)});\n"
+            # FMA and FMAAxBtC are a * b + c, FMAAxCtB is a * c + b, element by element (the reference prints
+            # warp::fma / fma_AxBtC / fma_AxCtB, Tyr/GPU/Codegen/AST.lean:196-206)
+            x, y, z = (s.a, s.c, s.b) if s.args[0] == "FMAAxCtB" else (s.a, s.b, s.c)
+            return f"{ind}wave::fma({I(s.dst)}, {I(x)}, {I(y)}, {I(z)});\n"
         if op in ("scalarMul", "scalarAdd"):
             f = "op_mul" if op == "scalarMul" else "op_add"
             return f"{ind}wave::scalar<{f}>({I(s.dst)}, {I(s.src)}, {_flt(s.scalar)});\n"
@@ -639,16 +651,18 @@ class _Emitter:
         if op == "binaryBroadcast":
             return f"{ind}wave::{s.axis.lower()}_broadcast<{BINARY[s.args[0]]}>({I(s.dst)}, {I(s.tile)}, {I(s.vec)});\n"
         if op in ("reduce", "reduceAccum"):
-            if s.axis == "Full":
-                raise UnsupportedStatement("full reductions have no gfx950 lowering yet")
             tail = f", {I(s.accum)}" if op == "reduceAccum" else ""
+            if s.axis == "Full":                         # every element of a vector or tile, left in every element of dst
+                if self.kind(s.dst) != "RV" or (op == "reduceAccum" and self.kind(s.src) != "RV"):
+                    raise UnsupportedStatement("a full reduction leaves its result in a register vector")
+                return f"{ind}wave::full_reduce<{REDUCE[s.args[0]]}>({I(s.dst)}, {I(s.src)}{tail});\n"
             return f"{ind}wave::{s.axis.lower()}_reduce<{REDUCE[s.args[0]]}>({I(s.dst)}, {I(s.src)}{tail});\n"
         if op == "outer":
             return f"{ind}wave::outer({I(s.dst)}, {I(s.a)}, {I(s.b)});\n"
         if op == "transpose":
-            if s.dst == s.src:
-                raise UnsupportedStatement("in-place transpose changes the tile's type; use a second tile")
             t, d = self.info[s.src], self.info[s.dst]
+            if s.dst == s.src and t.rows != t.cols:
+                raise UnsupportedStatement("an in-place transpose needs a square tile")
             if t.layout == d.layout:     # same layout kind on both sides: the data really moves, through LDS
                 return (f"{ind}{{\n{ind}  __shared__ st<{_cpp_type(t.dtype)}, {t.rows}, {t.cols}> {I(s.dst)}_tr;\n"
                         f"{ind}  wave::transpose({I(s.dst)}, {I(s.src)}, {I(s.dst)}_tr);\n{ind}}}\n")
@@ -958,10 +972,13 @@ class _Emitter:
             f"// the requested block becomes one 64-lane wave.  Returns 0, -2 (bad argument) or -1 (launch error).\n"
             f"extern \"C\" int tyr_launch_{name}({', '.join(cparams)}) {{\n" + "".join(setup) +
             f"  const uint64_t threads = block_x * block_y * block_z;\n"
-            f"  if (threads == 0 || grid_x * grid_y * grid_z == 0) return -2;\n"
-            f"  const unsigned waves = (unsigned)((threads + 31) / 32);\n" +
-            (f"  if (waves != {self.waves}) return -2;   // the program is compiled for a group of exactly {self.waves} waves\n"
-             if self.group else f"  if (waves > {self.max_waves}) return -2;\n") +
+            f"  if (threads == 0 || grid_x * grid_y * grid_z == 0) return -2;\n" +
+            (f"  // Every warp of the reference's block repeats the whole tile program, so the block shape does not change the\n"
+             f"  // result; here the program is cut into the row slices of a group of exactly {self.waves} waves, whatever was asked for.\n"
+             f"  const unsigned waves = {self.waves};\n"
+             if self.group else
+             f"  const unsigned waves = (unsigned)((threads + 31) / 32);\n"
+             f"  if (waves > {self.max_waves}) return -2;\n") +
             f"  hipLaunchKernelGGL({name}, dim3((unsigned)grid_x, (unsigned)grid_y, (unsigned)grid_z), dim3(64 * waves), "
             f"(size_t)shared_mem, static_cast<hipStream_t>(stream), {', '.join(args)});\n"
             f"  return hipGetLastError() == hipSuccess ? 0 : -1;\n}}\n")

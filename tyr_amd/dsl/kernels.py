@@ -649,6 +649,139 @@ def tkH100Fp8ScaledGemmFwd() -> Kernel:
     return k.build()
 
 
+def _causal_demo_attn_fwd(name: str, banner: str, with_lse: bool, explicit_softmax: bool) -> Kernel:
+    """The reference's three demonstration forwards with `makeCausal` share one shape: 64 x 64 tiles, four KV blocks, no
+    score scale, the per-tile causal mask with fill -1e10, and a score tile that is allocated once outside the loop and
+    *accumulated into* by every `mmaT s q k s` (it is never cleared: the scores of block j start from the probabilities of
+    block j-1, and from the tile's initial contents -- zeros in this lowering -- for block 0).
+      flashAttnFwdNew      Tyr/GPU/Kernels/FlashAttn.lean:26-95      onlineSoftmax / finalizeSoftmax macros
+      flashAttnFwdWithLse  Tyr/GPU/Kernels/FlashAttnBwd.lean:25-103  the same, plus LSE = ln(l) + m per row
+      flashAttnFwd         Tyr/GPU/Kernels/Examples.lean:93-144      running row max / row sum without rescaling O"""
+    k = KernelBuilder(name)
+    q_ptr = k.gptr("BFloat16", "q_ptr")
+    k_ptr = k.gptr("BFloat16", "k_ptr")
+    v_ptr = k.gptr("BFloat16", "v_ptr")
+    o_ptr = k.gptr("BFloat16", "o_ptr")
+    l_ptr = k.gptr("Float32", "l_ptr") if with_lse else None
+    k.kval("UInt64", "_seq_len")
+    k.kval("UInt64", "_head_dim")
+    if banner:
+        k.comment(banner)
+    coord = k.blockCoord2D()
+    q = k.allocRT("BFloat16", 64, 64)
+    kt = k.allocRT("BFloat16", 64, 64)
+    v = k.allocRT("BFloat16", 64, 64, "Col")
+    s_ = k.allocRT("Float32", 64, 64)
+    p = k.allocRT("BFloat16", 64, 64)
+    o = k.zeroRT("Float32", 64, 64)
+    if explicit_softmax:
+        rowMax = k.negInftyRV("Float32", 64)
+        rowSum = k.allocRV("Float32", 64)
+    else:
+        state = k.allocSoftmaxState("Float32", 64)
+    qS = k.allocST("BFloat16", 64, 64)
+    kS = k.allocST("BFloat16", 64, 64)
+    vS = k.allocST("BFloat16", 64, 64, "Col")
+    oS = k.allocST("BFloat16", 64, 64)
+    lS = k.allocSV("Float32", 64) if with_lse else None
+    k.loadGlobal(qS, q_ptr, coord)
+    k.sync()
+    k.load(q, qS)
+    with k.krange(0, 4) as kv:
+        k.loadGlobal(kS, k_ptr, coord.withRow(kv.id))
+        k.loadGlobal(vS, v_ptr, coord.withRow(kv.id))
+        k.sync()
+        k.load(kt, kS)
+        k.load(v, vS)
+        k.mmaT(s_, q, kt, s_)
+        k.makeCausal(s_, s_, -1e10)
+        if explicit_softmax:
+            k.rowMaxAccum(rowMax, s_, rowMax)
+            k.subCol(s_, s_, rowMax)
+            k.exp(s_, s_)
+            k.rowSumAccum(rowSum, s_, rowSum)
+        else:
+            k.onlineSoftmax(s_, o, state)
+        k.convert(p, s_)
+        k.mma(o, p, v, o)
+        k.sync()
+    if explicit_softmax:
+        k.divCol(o, o, rowSum)
+    else:
+        k.finalizeSoftmax(o, state)
+        if with_lse:
+            lse = k.computeLSE(state)
+    oBf16 = k.allocRT("BFloat16", 64, 64)
+    k.convert(oBf16, o)
+    k.store(oS, oBf16)
+    k.storeGlobal(o_ptr, oS, coord)
+    if with_lse:
+        k.storeVec(lS, lse)
+        k.storeVecGlobalRow(l_ptr, lS, coord)
+    return k.build()
+
+
+def flashAttnFwdNew() -> Kernel:
+    return _causal_demo_attn_fwd("flashAttnFwdNew", "=== FlashAttention Forward ===", False, False)
+
+
+def flashAttnFwdWithLse() -> Kernel:
+    return _causal_demo_attn_fwd("flashAttnFwdWithLse", "=== FlashAttention Forward (with LSE for backward) ===", True, False)
+
+
+def flashAttnFwd() -> Kernel:
+    return _causal_demo_attn_fwd("flashAttnFwd", "", False, True)
+
+
+def simpleGemmNew() -> Kernel:
+    """Tyr/GPU/Kernels/FlashAttn.lean:98-131 -- the test GEMM of that file: the program of `simpleGemm` under its own name."""
+    k = simpleGemm()
+    k.name = "simpleGemmNew"
+    return k
+
+
+def tkH100Fp8E4M3GemmFwd() -> Kernel:
+    """Tyr/GPU/Kernels/PrecisionGemm.lean:73-89 with GemmCommon.storeConvertedTile (GemmCommon.lean:58-69): the canonical
+    H100 FP8 surface, E4M3 x E4M3 -> f32 -> E4M3 on 64 x 256 output tiles, K = 512."""
+    k = KernelBuilder("tkH100Fp8E4M3GemmFwd")
+    aPtr = k.gptr("FP8E4M3", "aPtr")
+    bPtr = k.gptr("FP8E4M3", "bPtr")
+    cPtr = k.gptr("FP8E4M3", "cPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    accum, coord = _h100Fp8Accumulator(k, "=== H100 FP8 GEMM (E4M3 -> E4M3 epilogue) ===", aPtr, bPtr)
+    out = k.allocRT("FP8E4M3", 64, 256)
+    outShared = k.allocST("FP8E4M3", 64, 256)
+    k.convert(out, accum)
+    k.store(outShared, out)
+    k.storeGlobal(cPtr, outShared, coord)
+    return k.build()
+
+
+def tkB200Fp8E4M3Gemm1CtaFwd() -> Kernel:
+    """Tyr/GPU/Kernels/PrecisionGemm.lean:117-133 (accumulator :52-69): the Blackwell one-CTA surface, E4M3 x E4M3 -> f32 ->
+    bf16 on 128 x 256 output tiles, K = 512.  Nothing in the program is specific to that device; on gfx950 it is run by a
+    group of four waves with B read from LDS, like the H100 bf16 surface."""
+    k = KernelBuilder("tkB200Fp8E4M3Gemm1CtaFwd")
+    aPtr = k.gptr("FP8E4M3", "aPtr")
+    bPtr = k.gptr("FP8E4M3", "bPtr")
+    dPtr = k.gptr("BFloat16", "dPtr")
+    k.kval("UInt64", "m")
+    k.kval("UInt64", "n")
+    k.kval("UInt64", "k")
+    accum, coord = _tiledAccumulator(
+        k, "=== B200 FP8 GEMM (1 CTA) ===",
+        "ThunderKittens fp8_b200_gemm_1cta reduced to a typed 128x256 Blackwell-sized CTA mainloop",
+        aPtr, bPtr, "FP8E4M3", 128, 128, 256, 4)
+    out = k.allocRT("BFloat16", 128, 256)
+    outShared = k.allocST("BFloat16", 128, 256)
+    k.convert(out, accum)
+    k.store(outShared, out)
+    k.storeGlobal(dPtr, outShared, coord)
+    return k.build()
+
+
 # kernel name -> the reference definition it restates
 CITES = {
     "copy64x64": "Tyr/GPU/Kernels/Copy.lean:16-26 (runner Examples/GPU/RunCopy.lean:28)",
@@ -669,9 +802,16 @@ CITES = {
     "tkMhaH100LCFFwd64": "Tyr/GPU/Kernels/MhaH100LCF.lean:84-107 (run by a group of 2 waves, K and V read from LDS by the products)",
     "tkMhaH100LCFFwd128": "Tyr/GPU/Kernels/MhaH100LCF.lean:109-132 (run by a group of 2 waves, K and V read from LDS by the products)",
     "tkH100Bf16GemmFwd": "Tyr/GPU/Kernels/Bf16Gemm.lean:64-73 over GemmCommon.lean:22-69 (run by a group of 4 waves, B read from LDS by the products)",
+    "flashAttnFwdNew": "Tyr/GPU/Kernels/FlashAttn.lean:26-95",
+    "flashAttnFwdWithLse": "Tyr/GPU/Kernels/FlashAttnBwd.lean:25-103",
+    "flashAttnFwd": "Tyr/GPU/Kernels/Examples.lean:93-144",
+    "simpleGemmNew": "Tyr/GPU/Kernels/FlashAttn.lean:98-131",
+    "tkH100Fp8E4M3GemmFwd": "Tyr/GPU/Kernels/PrecisionGemm.lean:73-89 over GemmCommon.lean:22-69",
+    "tkB200Fp8E4M3Gemm1CtaFwd": "Tyr/GPU/Kernels/PrecisionGemm.lean:117-133 over GemmCommon.lean:22-69 (run by a group of 4 waves, B read from LDS by the products)",
 }
 ALL = (copy64x64, rotaryFwd, tkFusedLayerNormResidual1024, simpleGemm, gemmFp8E4M3Fwd, tkH100Fp8ScaledGemmFwd,
        tkFlashAttnFwd2Block, tkFlashAttnFwd2BlockLse,
        tkMhaH100Fwd2Block, tkMhaH100BwdPrep2Block, tkMhaH100Bwd2BlockPartials,
        tkFlashAttnFwd12Block, tkFlashAttnFwd12BlockLse, tkMhaH100Fwd12Block, tkMhaH100Bwd12BlockPartials,
-       tkMhaH100LCFFwd64, tkMhaH100LCFFwd128, tkH100Bf16GemmFwd)
+       tkMhaH100LCFFwd64, tkMhaH100LCFFwd128, tkH100Bf16GemmFwd,
+       flashAttnFwdNew, flashAttnFwdWithLse, flashAttnFwd, simpleGemmNew, tkH100Fp8E4M3GemmFwd, tkB200Fp8E4M3Gemm1CtaFwd)
