@@ -70,7 +70,8 @@ def test_online_softmax_macro_expands_to_the_reference_sequence():
 
 
 def test_emitted_text_goldens():
-    src = dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())
+    # statement by statement (the recognition of the online-softmax sequence switched off) ...
+    src = dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse(), fuse_online_softmax=False)
     for needle in [
         "__global__ __launch_bounds__(256) void tkFlashAttnFwd2BlockLse(gl<bf16> v0, gl<bf16> v1, gl<bf16> v2, "
         "gl<bf16> v3, gl<float> v4, uint64_t v5, uint64_t v6)",
@@ -89,6 +90,23 @@ def test_emitted_text_goldens():
     assert re.search(r"wave::gload\(v\d+_next, v1, coord\{\(int\)v\d+, \(int\)v\d+, \(int\)v\d+ \* 64, \(int\)v\d+ \* 64\}\);", src)
     # the vector store takes the row index as its unit coordinate (GlobalLayout.lean:343-349)
     assert re.search(r"wave::store\(v4, v\d+, \(int\)v\d+\);", src)
+    # ... and as emitted by default: the ten statements of `scalarMul` + `onlineSoftmax` (Macros.lean:121-147) become one call
+    # that leaves the same values in the same operands
+    fused = dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())
+    assert re.search(r"wave::online_softmax\(v\d+, v\d+, v\d+, v\d+, v\d+, v\d+, 0\.125f\);", fused)
+    for gone in ("wave::scalar<op_mul>(", "wave::row_reduce<op_max>(", "wave::col_broadcast<op_sub>(", "wave::row_reduce<op_add>("):
+        assert gone not in fused, gone
+    assert "wave::col_broadcast<op_div>(" in fused and "wave::unary<op_log>(" in fused        # finalizeSoftmax, computeLSE stay
+    # a sequence that differs in one operand is left alone
+    k = dsl.KernelBuilder("almost")
+    sc, o = k.zeroRT("Float32", 64, 64), k.zeroRT("Float32", 64, 64)
+    st_ = k.allocSoftmaxState("Float32", 64)
+    k.onlineSoftmax(sc, o, st_)
+    k.copyVec(st_.prevMax, st_.rowMax)
+    k.rowMaxAccum(st_.rowMax, sc, st_.rowMax)
+    k.subVec(st_.scale, st_.rowMax, st_.prevMax)             # operands swapped
+    text = dsl.emit_kernel(k.build())
+    assert text.count("wave::online_softmax(") == 1 and "wave::row_reduce<op_max>(" in text
 
 
 def test_register_vector_layouts_are_inferred():

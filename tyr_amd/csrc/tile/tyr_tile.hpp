@@ -707,6 +707,53 @@ __device__ __forceinline__ void outer(rt<T, R, C, layout::row>& dst, const rv<TV
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = from_f<T>(to_f(a.data[rb][0]) * to_f(b.data[cb][s]));
 }
 
+// ---------------------------------------------------------------- the online-softmax step as one operation
+// What the statement sequence of the reference's `onlineSoftmax` macro (Tyr/GPU/Codegen/Macros.lean:121-147), optionally
+// preceded by a multiplication of the scores by a positive constant, computes:
+//     prev = mx;  mx = max(mx, rowmax(c s));  scl = exp(prev - mx);  o *= scl;  sum *= scl;
+//     s = exp(c s - mx);  sum = rowsum(s) + sum
+// with the same values left in every operand.  Fused, the scale and the change to base 2 fold into one multiply-add per
+// score in front of the exponential instruction, and the accumulator is only rescaled when some row's maximum moved
+// (scl is exactly 1 otherwise).  The emitter substitutes this call where it recognises the sequence.
+template <int R, int C, int CO>
+__device__ __forceinline__ void online_softmax(rt<float, R, C, layout::row>& s, rt<float, R, CO, layout::row>& o,
+                                               rv<float, R, vlayout::align>& mx, rv<float, R, vlayout::align>& sum,
+                                               rv<float, R, vlayout::align>& prev, rv<float, R, vlayout::align>& scl, float c) {
+    constexpr float kLog2e = 1.4426950408889634f;
+#pragma unroll
+    for (int rb = 0; rb < R / 32; ++rb) {
+        float m = s.data[rb][0][0];
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int e = (cb == 0 ? 1 : 0); e < 16; ++e) m = fmaxf(m, s.data[rb][cb][e]);
+        m = fmaxf(m, xor32(m)) * c;                  // c > 0: the maximum of the scaled scores
+        const float old = mx.data[rb][0];
+        const float now = fmaxf(old, m);
+        const float f = __expf(old - now);
+        prev.data[rb][0] = old;
+        mx.data[rb][0] = now;
+        scl.data[rb][0] = f;
+        if (__builtin_amdgcn_ballot_w64(f != 1.0f) != 0) {
+#pragma unroll
+            for (int cb = 0; cb < CO / 32; ++cb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o.data[rb][cb][e] *= f;
+        }
+        const float c2 = c * kLog2e, m2 = now * kLog2e;
+        float acc = 0.0f;
+#pragma unroll
+        for (int cb = 0; cb < C / 32; ++cb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(s.data[rb][cb][e], c2, -m2));
+                s.data[rb][cb][e] = p;
+                acc += p;
+            }
+        sum.data[rb][0] = (acc + xor32(acc)) + sum.data[rb][0] * f;
+    }
+}
+
 // ---------------------------------------------------------------- full reductions and scans (vectors, tiles)
 // The reference's IR has a third axis, "Full" (Tyr/GPU/Codegen/AST.lean:54-63; printed as the unprefixed warp::max /
 // warp::sum / warp::cumsum, i.e. the vector forms): the reduction of every element, here left in every element of the
@@ -930,36 +977,49 @@ __device__ __forceinline__ void store(sv<T, N>& dst, const rv<T, NS, vlayout::al
 // Products whose B operand stays in LDS: its fragments are read as the product consumes them instead of
 // occupying a register tile (a 256x64 bf16 B would be 256 registers per lane).  The k <-> (lane half,
 // slot) map is that of the register tiles: slot e of half h of lane half g is k = 16h + 8(e/4) + 4g + e%4.
+// Fragments are requested `kStreamAhead` products ahead of their use (a small ring of registers) and the order is
+// pinned with scheduling fences: left alone the compiler, at its register limit in these kernels, puts each read directly
+// in front of its product and the wave sits out the LDS latency once per MFMA.
+constexpr int kStreamAhead = 4;
 // B as [N, K] rows (the DSL's mmaT): two 8-byte reads per fragment.
 template <int M, int N, int K>
 __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<bf16, M, K, layout::row>& a,
                                         const st<bf16, N, K>& b, const rt<float, M, N, layout::row>& c) {
+    constexpr int KS = K / 16, NF = (N / 32) * KS, P = kStreamAhead;
+    auto read = [&](int f) {
+        const bf16* p = b.at(32 * (f / KS) + lr(), 16 * (f % KS) + 4 * lg());
+        const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p), hi = *reinterpret_cast<const bf16x4*>(p + 8);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    bf16x8 ring[P];
 #pragma unroll
-    for (int nb = 0; nb < N / 32; ++nb) {
-        f32x16 acc[M / 32];
+    for (int f = 0; f < P - 1 && f < NF; ++f) ring[f] = read(f);
+    f32x16 acc[M / 32];
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
+    for (int f = 0; f < NF; ++f) {
+        const int nb = f / KS, ks = f % KS, kb = ks / 2, h = ks % 2;
+        if (f + P - 1 < NF) ring[(f + P - 1) % P] = read(f + P - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == 0) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+            for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll
-        for (int kb = 0; kb < K / 32; ++kb)
+                for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+        }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const bf16* p = b.at(32 * nb + lr(), 32 * kb + 16 * h + 4 * lg());
-                const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p), hi = *reinterpret_cast<const bf16x4*>(p + 8);
-                const bf16x8 fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int mb = 0; mb < M / 32; ++mb) {
+            bf16x8 fa;
 #pragma unroll
-                for (int mb = 0; mb < M / 32; ++mb) {
-                    bf16x8 fa;
+            for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
+            acc[mb] = mfma_32x32x16_bf16(ring[f % P], fa, acc[mb]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == KS - 1) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
-                    acc[mb] = mfma_32x32x16_bf16(fb, fa, acc[mb]);
-                }
-            }
+            for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+                for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+        }
     }
 }
 // E4M3 operands, B as [N, K] rows in LDS: a lane's 32 bytes of k for the 32x32x64 MFMA are the 16 bytes of its slots in two
@@ -968,40 +1028,52 @@ template <int M, int N, int K>
 __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<fp8e4m3, M, K, layout::row>& a,
                                         const st<fp8e4m3, N, K>& b, const rt<float, M, N, layout::row>& c) {
     static_assert(K % 64 == 0, "E4M3 products consume k in steps of 64");
+    constexpr int KS = K / 64, NF = (N / 32) * KS, P = 3;
+    auto read = [&](int f) {
+        i32x8 fb;
 #pragma unroll
-    for (int nb = 0; nb < N / 32; ++nb) {
-        f32x16 acc[M / 32];
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
+            for (int wd = 0; wd < 4; ++wd)
+                fb[4 * h + wd] = *reinterpret_cast<const int*>(b.at(32 * (f / KS) + lr(), 64 * (f % KS) + 32 * h + 8 * wd + 4 * lg()));
+        return fb;
+    };
+    i32x8 ring[P];
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+    for (int f = 0; f < P - 1 && f < NF; ++f) ring[f] = read(f);
+    f32x16 acc[M / 32];
 #pragma unroll
-        for (int kb = 0; kb < K / 32; kb += 2) {
-            i32x8 fb;
+    for (int f = 0; f < NF; ++f) {
+        const int nb = f / KS, kb = 2 * (f % KS);
+        if (f + P - 1 < NF) ring[(f + P - 1) % P] = read(f + P - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb == 0) {
+#pragma unroll
+            for (int mb = 0; mb < M / 32; ++mb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+        }
+#pragma unroll
+        for (int mb = 0; mb < M / 32; ++mb) {
+            i32x8 fa;
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int wd = 0; wd < 4; ++wd)
-                    fb[4 * h + wd] = *reinterpret_cast<const int*>(b.at(32 * nb + lr(), 32 * (kb + h) + 8 * wd + 4 * lg()));
+                for (int wd = 0; wd < 4; ++wd) {
+                    uint32_t ua = 0;
 #pragma unroll
-            for (int mb = 0; mb < M / 32; ++mb) {
-                i32x8 fa;
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int wd = 0; wd < 4; ++wd) {
-                        uint32_t ua = 0;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) ua |= (uint32_t)a.data[mb][kb + h][4 * wd + e].bits << (8 * e);
-                        fa[4 * h + wd] = (int)ua;
-                    }
-                acc[mb] = mfma_32x32x64_e4m3(fb, fa, acc[mb]);
-            }
+                    for (int e = 0; e < 4; ++e) ua |= (uint32_t)a.data[mb][kb + h][4 * wd + e].bits << (8 * e);
+                    fa[4 * h + wd] = (int)ua;
+                }
+            acc[mb] = mfma_32x32x64_e4m3(ring[f % P], fa, acc[mb]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb == 2 * (KS - 1)) {
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
+            for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+                for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+        }
     }
 }
 // B as [K, N] rows in LDS (the DSL's mma with a COL register tile): transposing reads, as load(rt col, st).
@@ -1010,32 +1082,42 @@ __device__ __forceinline__ void mma_AB(rt<float, M, N, layout::row>& d, const rt
                                        const st<bf16, K, N>& b, const rt<float, M, N, layout::row>& c) {
     const int i16 = lane() & 15, b16 = lane() >> 4;
     const int srow = 4 * (b16 >> 1) + (i16 >> 2), scol = 16 * (b16 & 1) + 4 * (i16 & 3);
+    constexpr int KS = K / 16, NF = (N / 32) * KS, P = kStreamAhead;
+    auto read = [&](int f) {
+        const int nb = f / KS, ks = f % KS;
+        const bf16x4 lo = ds_read_tr16(b.at(16 * ks + srow, 32 * nb + scol));
+        const bf16x4 hi = ds_read_tr16(b.at(16 * ks + 8 + srow, 32 * nb + scol));
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    bf16x8 ring[P];
 #pragma unroll
-    for (int nb = 0; nb < N / 32; ++nb) {
-        f32x16 acc[M / 32];
+    for (int f = 0; f < P - 1 && f < NF; ++f) ring[f] = read(f);
+    f32x16 acc[M / 32];
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
+    for (int f = 0; f < NF; ++f) {
+        const int nb = f / KS, ks = f % KS, kb = ks / 2, h = ks % 2;
+        if (f + P - 1 < NF) ring[(f + P - 1) % P] = read(f + P - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == 0) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+            for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll
-        for (int kb = 0; kb < K / 32; ++kb)
+                for (int e = 0; e < 16; ++e) acc[mb][e] = c.data[mb][nb][e];
+        }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const bf16x4 lo = ds_read_tr16(b.at(32 * kb + 16 * h + srow, 32 * nb + scol));
-                const bf16x4 hi = ds_read_tr16(b.at(32 * kb + 16 * h + 8 + srow, 32 * nb + scol));
-                const bf16x8 fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int mb = 0; mb < M / 32; ++mb) {
+            bf16x8 fa;
 #pragma unroll
-                for (int mb = 0; mb < M / 32; ++mb) {
-                    bf16x8 fa;
+            for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
+            acc[mb] = mfma_32x32x16_bf16(ring[f % P], fa, acc[mb]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == KS - 1) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) fa[e] = a.data[mb][kb][8 * h + e];
-                    acc[mb] = mfma_32x32x16_bf16(fb, fa, acc[mb]);
-                }
-            }
+            for (int mb = 0; mb < M / 32; ++mb)
 #pragma unroll
-        for (int mb = 0; mb < M / 32; ++mb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+                for (int e = 0; e < 16; ++e) d.data[mb][nb][e] = acc[mb][e];
+        }
     }
 }
 

@@ -500,8 +500,10 @@ def wave_group_plan(kernel: Kernel, rv_layout: Dict[VarId, str]):
 
 class _Emitter:
     def __init__(self, kernel: Kernel, max_waves: int = 4, hazard_barriers: bool = True,
-                 prefetch_global_loads: bool = True, share_lds: bool = True, wave_group=None):
+                 prefetch_global_loads: bool = True, share_lds: bool = True, wave_group=None,
+                 fuse_online_softmax: bool = True):
         self.k = kernel
+        self.fuse_online_softmax = fuse_online_softmax
         self.info: Dict[VarId, Stmt] = {}
         for s in walk(kernel.body):
             if s.op in ("declRT", "declST", "declRV", "declSV", "declGPtr", "declKVal"):
@@ -818,7 +820,7 @@ class _Emitter:
                "".join(request(t, ind2 + "    ") for t in pre) + f"{ind2}  }}\n{ind2}}}\n")
         placed = False
         remaining = len(pre)
-        for t in loop.body:
+        for t in self.fused(loop.body):
             if id(t) in frag:
                 if id(t) in self.barrier_before:
                     out += f"{ind2}wave::sync();  // inserted: a shared tile is overwritten below after other waves read it\n"
@@ -859,7 +861,76 @@ class _Emitter:
         return out
 
     def body(self, stmts, ind: str) -> str:
-        return "".join(self.one(s, ind) for s in stmts)
+        return "".join(self.one(s, ind) for s in self.fused(stmts))
+
+    # ------------------------------------------------------------------ recognised statement sequences
+    def fused(self, stmts):
+        """The statement list with every occurrence of the online-softmax step (the expansion of the reference's
+        `onlineSoftmax` macro, Macros.lean:121-147, with the score scaling in front of it if there is one) replaced by one
+        call of `wave::online_softmax`.  Only register tiles and vectors are involved, so no barrier analysis refers to
+        the statements that disappear."""
+        if not self.fuse_online_softmax:
+            return list(stmts)
+        L, out, i = list(stmts), [], 0
+        while i < len(L):
+            m = self._match_online_softmax(L, i)
+            if m is None:
+                out.append(L[i])
+                i += 1
+            else:
+                out.append(m[0])
+                i = m[1]
+        return out
+
+    def _match_online_softmax(self, L, i):
+        def nxt(j):                                      # next statement that is not a comment
+            while j < len(L) and L[j].op == "comment":
+                j += 1
+            return j
+        c, j = 1.0, nxt(i)
+        if j < len(L) and L[j].op == "scalarMul" and L[j].dst == L[j].src and L[j].scalar > 0:
+            c, S, j = L[j].scalar, L[j].dst, nxt(j + 1)
+        else:
+            S = None
+        got = []
+        for _ in range(9):
+            if j >= len(L):
+                return None
+            got.append(L[j])
+            j = nxt(j + 1)
+        s1, s2, s3, s4, s5, s6, s7, s8, s9 = got
+        try:
+            ok = (s1.op == "unary" and s1.args[0] == "Copy" and
+                  s2.op == "reduceAccum" and s2.args[0] == "Max" and s2.axis == "Row" and s2.dst == s2.accum == s1.src and
+                  (S is None or s2.src == S) and
+                  s3.op == "binary" and s3.args[0] == "Sub" and s3.a == s1.dst and s3.b == s2.dst and
+                  s4.op == "unary" and s4.args[0] == "Exp" and s4.dst == s4.src == s3.dst and
+                  s5.op == "binaryBroadcast" and s5.args[0] == "Mul" and s5.axis == "Col" and s5.dst == s5.tile and s5.vec == s3.dst and
+                  s6.op == "binary" and s6.args[0] == "Mul" and s6.dst == s6.a and s6.b == s3.dst and
+                  s7.op == "binaryBroadcast" and s7.args[0] == "Sub" and s7.axis == "Col" and s7.dst == s7.tile == s2.src and s7.vec == s2.dst and
+                  s8.op == "unary" and s8.args[0] == "Exp" and s8.dst == s8.src == s2.src and
+                  s9.op == "reduceAccum" and s9.args[0] == "Sum" and s9.axis == "Row" and s9.dst == s9.accum == s6.dst and s9.src == s2.src)
+        except AttributeError:
+            return None
+        if not ok:
+            return None
+        S, O, mx, sm, prev, scl = s2.src, s5.dst, s2.dst, s6.dst, s1.dst, s3.dst
+        if len({S, O}) != 2 or len({mx, sm, prev, scl}) != 4:
+            return None
+        for t in (S, O):
+            d = self.info.get(t)
+            if d is None or d.op != "declRT" or d.dtype != "Float32" or d.layout != "Row" or t in self.streamed:
+                return None
+        for v in (mx, sm, prev, scl):
+            d = self.info.get(v)
+            if d is None or d.op != "declRV" or d.dtype != "Float32" or self.rv_layout.get(v) != "align":
+                return None
+        if len({(v in self.split) for v in (S, O, mx, sm, prev, scl)}) != 1:
+            return None
+        from .ir import stmt as mk
+        code = (f"wave::online_softmax({S.ident}, {O.ident}, {mx.ident}, {sm.ident}, {prev.ident}, {scl.ident}, {_flt(c)});"
+                f"  // the online-softmax step{' with its score scale' if c != 1.0 else ''}, fused")
+        return mk("raw", code), j
 
     # ------------------------------------------------------------------ wave groups: who reads whose share
     def _group_rw(self, s: Stmt):
@@ -1058,10 +1129,10 @@ def emit_header(kernels: List[Kernel], cites: Dict[str, str]) -> str:
 
 
 def emit_kernel(kernel: Kernel, hazard_barriers: bool = True, prefetch_global_loads: bool = True,
-                share_lds: bool = True) -> str:
+                share_lds: bool = True, fuse_online_softmax: bool = True) -> str:
     """Device code of one kernel (no includes)."""
     return _Emitter(kernel, hazard_barriers=hazard_barriers, prefetch_global_loads=prefetch_global_loads,
-                    share_lds=share_lds).kernel_text()
+                    share_lds=share_lds, fuse_online_softmax=fuse_online_softmax).kernel_text()
 
 
 def emit_translation_unit(kernels: List[Kernel]) -> str:
