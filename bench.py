@@ -52,7 +52,7 @@ PEAK = {"mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "hbm": 8000.0}   # TFLOP/s, TFL
 # read for the 1 GiB copy of --workload copy_1gib (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the raw
 # figures are kept as text under profiles/.
 BWD_KERNELS = "flash_attn_bwd_dq_kernel<128,true> + flash_attn_bwd_dkv_kernel<128,true>"
-TRAFFIC = {"attn_fwd_causal": 1_119_610_880 + 274_726_912, "gqa_decode": 1_090_820_096 + 270_336,
+TRAFFIC = {"attn_fwd_causal": 1_079_701_504 + 289_406_976, "gqa_decode": 1_090_820_096 + 270_336,
            "gemm_bf16": 202_589_594 + 33_554_432, "gemm_fp8": 810_477_568 + 136_314_880,
            # both backward kernels: dQ (1,713,229,824 + 276,824,064) + dK/dV (1,082,617,856 + 536,870,912)
            "attn_bwd_causal": 1_647_249_408 + 276_824_064 + 1_082_636_288 + 536_870_912,
@@ -62,7 +62,8 @@ TRAFFIC = {"attn_fwd_causal": 1_119_610_880 + 274_726_912, "gqa_decode": 1_090_8
            "decode_rope_append_kernel + gqa_decode_split_kernel<8>": 423_680 + 393_216 + 1_090_152_448 + 270_336,
            "gqa_decode_split4": 1_085_655_040 + 2_228_224 + 2_403_328 + 294_912,       # split pass + combine pass
            "gqa_decode_small_batch": 542_947_328 + 589_824 + 601_088 + 36_864,
-           "dsl_simple_gemm": 77_063_987 + 268_435_456, "dsl_h100_gemm": 37_877_146 + 134_217_728}
+           "dsl_simple_gemm": 77_063_987 + 268_435_456, "dsl_h100_gemm": 39_013_376 + 134_217_728,
+           "dsl_lcf_attn": 655_022_080 + 50_331_648}
 
 
 def _events(torch, n):
@@ -179,17 +180,21 @@ def wl_attn(torch, tyr, steps, warmup, cpu, parity):
     wall, ms = time_steps(torch, fn, steps, warmup)
     flop = 4.0 * B * H * N * N * D / 2.0
     tf = flop / (ms * 1e-3) / 1e12
-    # the two launch shapes of the forward, timed alternately after the headline's timed region (same box, same run)
+    # The two launch shapes of the forward, timed alternately after the headline's timed region (same box, same run).  A
+    # comparison leg: it runs with the output check only, so that a profile taken with --no-parity holds the launches of the
+    # default shape and nothing else.
     from tyr_amd import _lib
     L = _lib.load()
     default_shape = L.tyr_hip_flash_attn_fwd_persistent(0)
-    pair = {"per_job": [], "persistent": []}
-    for _ in range(3):
-        for name, on in (("per_job", 0), ("persistent", 1)):
-            L.tyr_hip_flash_attn_fwd_persistent(on)
-            pair[name].append(time_steps(torch, fn, steps, 2)[1])
     L.tyr_hip_flash_attn_fwd_persistent(default_shape)
-    fn()                                            # `out` holds a launch of the default shape again
+    pair = {"per_job": [], "persistent": []}
+    if parity:
+        for _ in range(3):
+            for name, on in (("per_job", 0), ("persistent", 1)):
+                L.tyr_hip_flash_attn_fwd_persistent(on)
+                pair[name].append(time_steps(torch, fn, steps, 2)[1])
+        L.tyr_hip_flash_attn_fwd_persistent(default_shape)
+        fn()                                        # `out` holds a launch of the default shape again
     res = {
         "metric": "attn fwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "wall_ms_per_step": wall,
         "dtype": "bf16",
@@ -197,7 +202,7 @@ def wl_attn(torch, tyr, steps, warmup, cpu, parity):
                    "flop_convention": "4*B*H*N^2*D/2 (causal half)", "scale": "1/sqrt(128)",
                    "inputs": "torch.manual_seed(0); Q, K, V = randn on the host in that order -> bf16 -> device",
                    "launch_shape": "persistent" if default_shape else "per_job",
-                   "launch_shapes_ms": {k_: round(sorted(v_)[1], 5) for k_, v_ in pair.items()}},
+                   "launch_shapes_ms": {k_: round(sorted(v_)[1], 5) for k_, v_ in pair.items()} if parity else None},
         "roofline": _mfma_roofline(torch, "mfma_bf16", "flash_attn_fwd_kernel<128,true>", tf, TRAFFIC["attn_fwd_causal"]),
     }
     if parity:

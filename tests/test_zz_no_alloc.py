@@ -77,3 +77,50 @@ def test_static_decode_rejects_oversized_request():
     rc = L_.tyr_hip_gqa_decode_static(t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), None,
                                       B, Hq, Hkv, Lmax, D, Lmax, 0.1, splits, None)
     assert rc == -5 and b"workspace" in L_.tyr_hip_strerror(rc)
+
+
+def _free_device_bytes():
+    free, _total = torch.cuda.mem_get_info()
+    return free
+
+
+def test_static_decode_allocates_nothing_and_replays_from_a_captured_graph():
+    """The entry point takes no memory from the device or from the caching allocator (outputs are the caller's), and --
+    after one warm-up call, which resolves the address of the static array -- it can be recorded into a HIP graph: three
+    replays with eager work in between, each equal to the eager result of the workspace entry point."""
+    from tyr_amd import _lib
+    L_ = _lib.load()
+    B, Hq, Hkv, Lmax, D, splits = 2, 8, 2, 900, 128, 4
+    sc = 1 / math.sqrt(D)
+    q, = lt.make_inputs(940, (B, Hq, 1, D))
+    k, v = lt.make_inputs(941, (B, Hkv, Lmax, D), (B, Hkv, Lmax, D))
+    q, k, v = q.cuda(), k.cuda(), v.cuda()
+    (o_s, lse_s), (o_w, lse_w) = _call_pair(L_, q, k, v, splits, Lmax)           # warm-up + reference result
+    o = torch.zeros_like(q)
+    lse = torch.zeros((B, Hq), device="cuda")
+    torch.cuda.synchronize()
+
+    def call(stream):
+        rc = L_.tyr_hip_gqa_decode_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                          B, Hq, Hkv, Lmax, D, Lmax, sc, splits, stream)
+        assert rc == 0, L_.tyr_hip_strerror(rc)
+
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _free_device_bytes())
+    for _ in range(3):
+        call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _free_device_bytes())
+    assert before == after, (before, after)
+    assert torch.equal(o, o_w) and torch.equal(lse, lse_w)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        o.zero_(); lse.zero_()                                                   # eager work between the replays
+        junk = torch.full((1 << 18,), float(replay), device="cuda")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_w) and torch.equal(lse, lse_w), replay
+        del junk
