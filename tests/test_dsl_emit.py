@@ -76,7 +76,8 @@ def test_emitted_text_goldens():
         "__global__ __launch_bounds__(256) void tkFlashAttnFwd2BlockLse(gl<bf16> v0, gl<bf16> v1, gl<bf16> v2, "
         "gl<bf16> v3, gl<float> v4, uint64_t v5, uint64_t v6)",
         "rt<bf16, 64, 64, layout::col>",                       # v is a Col tile
-        "st<bf16, 64, 64>& v", "unsigned char tyr_lds_pool[18432];",     # Q / O tile over the K tile, V tile beside them
+        "st<bf16, 64, 64>& v", "st<bf16, 64, 64, 32>& v",                # the V tile (read transposed) has the wider row pad
+            "unsigned char tyr_lds_pool[19456];",                             # Q / O tile over the V tile, K tile beside them
         "__shared__ sv<float, 64>",
         "wave::mma_ABt(", "wave::mma_AB(",
         "wave::scalar<op_mul>(", "0.125f);",
@@ -269,14 +270,14 @@ def test_global_tiles_of_a_loop_are_requested_one_iteration_ahead():
 
 def test_lds_tiles_with_disjoint_live_ranges_share_storage():
     # simpleGemm: the f32 staging tile of the result is only used after the k loop, its A and B tiles
-    # only inside it -- one pool of 18,432 bytes instead of 35,840, i.e. twice the workgroups per CU
+    # only inside it -- one pool of 19,456 bytes instead of 36,864, i.e. twice the workgroups per CU
     src = dsl.emit_kernel(kernels.simpleGemm())
-    assert "unsigned char tyr_lds_pool[18432];" in src
-    assert src.count("tyr_lds_pool + 0)") == 2 and "tyr_lds_pool + 9216)" in src
+    assert "unsigned char tyr_lds_pool[19456];" in src
+    assert src.count("tyr_lds_pool + 0)") == 2 and "tyr_lds_pool + 10240)" in src
     plain = dsl.emit_kernel(kernels.simpleGemm(), share_lds=False)
     assert "tyr_lds_pool" not in plain and plain.count("__shared__ st<") == 3
     # tiles that are live together never overlap: every pair of tiles used in one loop is disjoint
-    from tyr_amd.dsl.emit import lds_plan
+    from tyr_amd.dsl.emit import lds_plan, st_bytes
     for make in kernels.ALL:
         k = make()
         name = k.name
@@ -284,7 +285,7 @@ def test_lds_tiles_with_disjoint_live_ranges_share_storage():
         decl = {t.v: t for t in walk(k.body) if t.op == "declST"}
         for body in [t.body for t in walk(k.body) if t.op in ("forLoop", "forLoopVal")]:
             used = {a for t in walk(body) for a in t.args if isinstance(a, VarId) and a in plan}
-            spans = sorted((plan[v], plan[v] + decl[v].rows * decl[v].cols) for v in used)
+            spans = sorted((plan[v], plan[v] + st_bytes(decl[v])) for v in used)
             assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), (name, spans)
     # a kernel whose tiles are all live together keeps its plain declarations
     assert "tyr_lds_pool" not in dsl.emit_kernel(kernels.tkFusedLayerNormResidual1024())
@@ -292,10 +293,12 @@ def test_lds_tiles_with_disjoint_live_ranges_share_storage():
     # K tile.  That costs one barrier in front of the loop (every wave has Q in registers before K(0) is written) and none
     # inside it; a plan that would put a barrier into a loop is dropped instead.
     att = dsl.emit_kernel(kernels.tkFlashAttnFwd2BlockLse())
-    assert "unsigned char tyr_lds_pool[18432];" in att and att.count("// inserted:") == 1
+    assert "unsigned char tyr_lds_pool[19456];" in att and att.count("// inserted:") == 1
     assert att.index("// inserted:") < att.index("for (int")
     lcf = dsl.emit_kernel(kernels.tkMhaH100LCFFwd128())
-    assert "unsigned char tyr_lds_pool[69632];" in lcf               # 104,448 bytes as separate tiles: two workgroups per CU now
+    assert "unsigned char tyr_lds_pool[71680];" in lcf               # 108,544 bytes as separate tiles: two workgroups per CU now
+    # tiles read with the transposing LDS read (column-major operands of 2-byte elements) get 32 bytes of row padding, the others 16
+    assert "st<bf16, 128, 128, 32>& v" in lcf and "st<bf16, 128, 128>& v" in lcf
     assert lcf.index("// inserted: a shared tile is overwritten") < lcf.index("for (int")
 
 

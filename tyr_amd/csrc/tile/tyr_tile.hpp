@@ -67,10 +67,13 @@ struct rt {
 
 // LDS tile, row-major, rows padded by 16 bytes (32 lanes reading one column chunk of 32
 // consecutive rows then spread over the banks).
-template <typename T, int R, int C>
+// PAD: bytes of padding behind every row (a multiple of 16, so that rows stay 16-byte aligned).  Which value keeps the banks
+// apart depends on how the tile is read; the emitter chooses it per tile.
+template <typename T, int R, int C, int PAD = 16>
 struct st {
+    static_assert(PAD % 16 == 0, "rows stay 16-byte aligned");
     typedef T dtype;
-    static constexpr int rows = R, cols = C, pitch = C + 16 / (int)sizeof(T);
+    static constexpr int rows = R, cols = C, pitch = C + PAD / (int)sizeof(T);
     T data[R * pitch];
     __device__ __forceinline__ T* at(int r, int c) { return data + r * pitch + c; }
     __device__ __forceinline__ const T* at(int r, int c) const { return data + r * pitch + c; }
@@ -176,8 +179,8 @@ namespace wave {
 using namespace detail;
 
 // ---------------------------------------------------------------- global <-> LDS
-template <typename T, int R, int C>
-__device__ __forceinline__ void load(st<T, R, C>& dst, const gl<T>& src, coord at) {
+template <typename T, int R, int C, int PAD>
+__device__ __forceinline__ void load(st<T, R, C, PAD>& dst, const gl<T>& src, coord at) {
     constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
     static_assert(C % VEC == 0 && (R * CPR) % 64 == 0, "tile is not a whole number of 16-byte pieces per lane");
 #pragma unroll
@@ -205,8 +208,8 @@ __device__ __forceinline__ void gload(gfrag<T, R, C>& dst, const gl<T>& src, coo
         dst.v[k] = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
     }
 }
-template <typename T, int R, int C>
-__device__ __forceinline__ void sstore(st<T, R, C>& dst, const gfrag<T, R, C>& src) {
+template <typename T, int R, int C, int PAD>
+__device__ __forceinline__ void sstore(st<T, R, C, PAD>& dst, const gfrag<T, R, C>& src) {
     typedef gfrag<T, R, C> F;
 #pragma unroll
     for (int k = 0; k < F::N; ++k) {
@@ -215,8 +218,8 @@ __device__ __forceinline__ void sstore(st<T, R, C>& dst, const gfrag<T, R, C>& s
     }
     wave_fence();
 }
-template <typename T, int R, int C>
-__device__ __forceinline__ void store(const gl<T>& dst, const st<T, R, C>& src, coord at) {
+template <typename T, int R, int C, int PAD>
+__device__ __forceinline__ void store(const gl<T>& dst, const st<T, R, C, PAD>& src, coord at) {
     constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
     static_assert(C % VEC == 0 && (R * CPR) % 64 == 0, "tile is not a whole number of 16-byte pieces per lane");
     wave_fence();
@@ -258,8 +261,8 @@ __device__ __forceinline__ void store(const gl<T>& dst, const sv<T, N>& src, coo
 }
 
 // atomic accumulation into global memory (f32).  Every wave that executes the statement adds.
-template <int R, int C>
-__device__ __forceinline__ void store_add(const gl<float>& dst, const st<float, R, C>& src, coord at) {
+template <int R, int C, int PAD>
+__device__ __forceinline__ void store_add(const gl<float>& dst, const st<float, R, C, PAD>& src, coord at) {
     wave_fence();
 #pragma unroll
     for (int k = 0; k < R * C / 64; ++k) {
@@ -286,8 +289,8 @@ __device__ __forceinline__ void store_add(const gl<float>& dst, const sv<float, 
 namespace detail {
 // The four slots 4q .. 4q+3 of a ROW tile are four consecutive columns of one row: one 4-element access.
 template <typename T> struct quad { T v[4]; } __attribute__((aligned(sizeof(T) * 4 <= 16 ? sizeof(T) * 4 : 16)));
-template <typename T, int RS, int R, int C>
-__device__ __forceinline__ void load_rows(rt<T, RS, C, layout::row>& dst, const st<T, R, C>& src, int row0) {
+template <typename T, int RS, int R, int C, int PAD>
+__device__ __forceinline__ void load_rows(rt<T, RS, C, layout::row>& dst, const st<T, R, C, PAD>& src, int row0) {
 #pragma unroll
     for (int rb = 0; rb < RS / 32; ++rb)
 #pragma unroll
@@ -299,8 +302,8 @@ __device__ __forceinline__ void load_rows(rt<T, RS, C, layout::row>& dst, const 
                 for (int x = 0; x < 4; ++x) dst.data[rb][cb][4 * q + x] = v.v[x];
             }
 }
-template <typename T, int RS, int R, int C>
-__device__ __forceinline__ void store_rows(st<T, R, C>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
+template <typename T, int RS, int R, int C, int PAD>
+__device__ __forceinline__ void store_rows(st<T, R, C, PAD>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
 #pragma unroll
     for (int rb = 0; rb < RS / 32; ++rb)
 #pragma unroll
@@ -314,8 +317,8 @@ __device__ __forceinline__ void store_rows(st<T, R, C>& dst, const rt<T, RS, C, 
             }
 }
 }  // namespace detail
-template <typename T, int R, int C, layout L>
-__device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src) {
+template <typename T, int R, int C, layout L, int PAD>
+__device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C, PAD>& src) {
     typedef rt<T, R, C, L> RT;
     if constexpr (L == layout::row) {
         detail::load_rows(dst, src, 0);
@@ -325,8 +328,8 @@ __device__ __forceinline__ void load(rt<T, R, C, L>& dst, const st<T, R, C>& src
 }
 // COL tiles of 2-byte elements: a lane wants 4 consecutive rows of one column per slot group, which is
 // what the transposing LDS read delivers (16 lanes x 8 bytes along 4 rows in, 4 rows of one column out).
-template <int R, int C>
-__device__ __forceinline__ void load(rt<bf16, R, C, layout::col>& dst, const st<bf16, R, C>& src) {
+template <int R, int C, int PAD>
+__device__ __forceinline__ void load(rt<bf16, R, C, layout::col>& dst, const st<bf16, R, C, PAD>& src) {
     const int i16 = lane() & 15, b16 = lane() >> 4;
     const int srow = 4 * (b16 >> 1) + (i16 >> 2), scol = 16 * (b16 & 1) + 4 * (i16 & 3);   // this lane as a source
 #pragma unroll
@@ -340,8 +343,8 @@ __device__ __forceinline__ void load(rt<bf16, R, C, layout::col>& dst, const st<
                 for (int x = 0; x < 4; ++x) dst.data[rb][cb][4 * q + x] = v[x];
             }
 }
-template <typename T, int R, int C, layout L>
-__device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, R, C, L>& src) {
+template <typename T, int R, int C, layout L, int PAD>
+__device__ __forceinline__ void store(st<T, R, C, PAD>& dst, const rt<T, R, C, L>& src) {
     typedef rt<T, R, C, L> RT;
     if constexpr (L == layout::row) {
         detail::store_rows(dst, src, 0);
@@ -542,16 +545,16 @@ __device__ __forceinline__ void transpose(rt<T, C, R, layout::row>& dst, const r
             for (int s = 0; s < 16; ++s) dst.data[cb][rb][s] = src.data[rb][cb][s];
 }
 // Transpose that keeps the layout kind: through an LDS tile of the source's shape.
-template <typename T, int R, int C, layout L>
-__device__ __forceinline__ void transpose(rt<T, C, R, L>& dst, const rt<T, R, C, L>& src, st<T, R, C>& scratch) {
+template <typename T, int R, int C, layout L, int PAD>
+__device__ __forceinline__ void transpose(rt<T, C, R, L>& dst, const rt<T, R, C, L>& src, st<T, R, C, PAD>& scratch) {
     store(scratch, src);
     typedef rt<T, C, R, L> RT;
     TYR_TILE_FOR_BLOCKS(RT) dst.data[rb][cb][s] = *scratch.at(col_of<L>(cb, s), row_of<L>(rb, s));
     wave_fence();
 }
 // Same matrix, other layout: through an LDS tile the caller provides.
-template <typename T, int R, int C, layout LD, layout LS>
-__device__ __forceinline__ void swap_layout(rt<T, R, C, LD>& dst, const rt<T, R, C, LS>& src, st<T, R, C>& scratch) {
+template <typename T, int R, int C, layout LD, layout LS, int PAD>
+__device__ __forceinline__ void swap_layout(rt<T, R, C, LD>& dst, const rt<T, R, C, LS>& src, st<T, R, C, PAD>& scratch) {
     store(scratch, src);
     load(dst, scratch);
     wave_fence();
@@ -901,8 +904,8 @@ __device__ __forceinline__ void sync() { __syncthreads(); }
 __device__ __forceinline__ int index() { return (int)(threadIdx.x >> 6); }
 
 // global <-> LDS, the group sharing the tile: wave `part` of `nparts` moves its share of the rows
-template <typename T, int R, int C>
-__device__ __forceinline__ void load_part(st<T, R, C>& dst, const gl<T>& src, coord at, int part, int nparts) {
+template <typename T, int R, int C, int PAD>
+__device__ __forceinline__ void load_part(st<T, R, C, PAD>& dst, const gl<T>& src, coord at, int part, int nparts) {
     constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
     static_assert(C % VEC == 0, "rows are whole 16-byte pieces");
     for (int idx = part * 64 + lane(); idx < R * CPR; idx += 64 * nparts) {
@@ -911,8 +914,8 @@ __device__ __forceinline__ void load_part(st<T, R, C>& dst, const gl<T>& src, co
     }
     wave_fence();
 }
-template <typename T, int R, int C>
-__device__ __forceinline__ void store_part(const gl<T>& dst, const st<T, R, C>& src, coord at, int part, int nparts) {
+template <typename T, int R, int C, int PAD>
+__device__ __forceinline__ void store_part(const gl<T>& dst, const st<T, R, C, PAD>& src, coord at, int part, int nparts) {
     constexpr int VEC = 16 / (int)sizeof(T), CPR = C / VEC;
     static_assert(C % VEC == 0, "rows are whole 16-byte pieces");
     wave_fence();
@@ -939,8 +942,8 @@ __device__ __forceinline__ void gload_part(gfrag_part<T, R, C, W>& dst, const gl
         dst.v[k] = *reinterpret_cast<const u32x4*>(src.at(at.b, at.d, at.r + r, at.c + c));
     }
 }
-template <typename T, int R, int C, int W>
-__device__ __forceinline__ void sstore_part(st<T, R, C>& dst, const gfrag_part<T, R, C, W>& src, int part) {
+template <typename T, int R, int C, int W, int PAD>
+__device__ __forceinline__ void sstore_part(st<T, R, C, PAD>& dst, const gfrag_part<T, R, C, W>& src, int part) {
     typedef gfrag_part<T, R, C, W> F;
 #pragma unroll
     for (int k = 0; k < F::N; ++k) {
@@ -950,13 +953,13 @@ __device__ __forceinline__ void sstore_part(st<T, R, C>& dst, const gfrag_part<T
     wave_fence();
 }
 // a wave's row slice of an LDS tile / vector <-> registers
-template <typename T, int RS, int R, int C>
-__device__ __forceinline__ void load(rt<T, RS, C, layout::row>& dst, const st<T, R, C>& src, int row0) {
+template <typename T, int RS, int R, int C, int PAD>
+__device__ __forceinline__ void load(rt<T, RS, C, layout::row>& dst, const st<T, R, C, PAD>& src, int row0) {
     static_assert(RS <= R, "a slice is no taller than its tile");
     detail::load_rows(dst, src, row0);
 }
-template <typename T, int RS, int R, int C>
-__device__ __forceinline__ void store(st<T, R, C>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
+template <typename T, int RS, int R, int C, int PAD>
+__device__ __forceinline__ void store(st<T, R, C, PAD>& dst, const rt<T, RS, C, layout::row>& src, int row0) {
     static_assert(RS <= R, "a slice is no taller than its tile");
     detail::store_rows(dst, src, row0);
     wave_fence();
@@ -982,9 +985,9 @@ __device__ __forceinline__ void store(sv<T, N>& dst, const rv<T, NS, vlayout::al
 // in front of its product and the wave sits out the LDS latency once per MFMA.
 constexpr int kStreamAhead = 4;
 // B as [N, K] rows (the DSL's mmaT): two 8-byte reads per fragment.
-template <int M, int N, int K>
+template <int M, int N, int K, int PAD>
 __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<bf16, M, K, layout::row>& a,
-                                        const st<bf16, N, K>& b, const rt<float, M, N, layout::row>& c) {
+                                        const st<bf16, N, K, PAD>& b, const rt<float, M, N, layout::row>& c) {
     constexpr int KS = K / 16, NF = (N / 32) * KS, P = kStreamAhead;
     auto read = [&](int f) {
         const bf16* p = b.at(32 * (f / KS) + lr(), 16 * (f % KS) + 4 * lg());
@@ -1024,9 +1027,9 @@ __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const r
 }
 // E4M3 operands, B as [N, K] rows in LDS: a lane's 32 bytes of k for the 32x32x64 MFMA are the 16 bytes of its slots in two
 // adjacent 32-column blocks (the map of the register tiles), i.e. eight 4-byte pieces at columns 32kb + 8q + 4g.
-template <int M, int N, int K>
+template <int M, int N, int K, int PAD>
 __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const rt<fp8e4m3, M, K, layout::row>& a,
-                                        const st<fp8e4m3, N, K>& b, const rt<float, M, N, layout::row>& c) {
+                                        const st<fp8e4m3, N, K, PAD>& b, const rt<float, M, N, layout::row>& c) {
     static_assert(K % 64 == 0, "E4M3 products consume k in steps of 64");
     constexpr int KS = K / 64, NF = (N / 32) * KS, P = 3;
     auto read = [&](int f) {
@@ -1077,9 +1080,9 @@ __device__ __forceinline__ void mma_ABt(rt<float, M, N, layout::row>& d, const r
     }
 }
 // B as [K, N] rows in LDS (the DSL's mma with a COL register tile): transposing reads, as load(rt col, st).
-template <int M, int N, int K>
+template <int M, int N, int K, int PAD>
 __device__ __forceinline__ void mma_AB(rt<float, M, N, layout::row>& d, const rt<bf16, M, K, layout::row>& a,
-                                       const st<bf16, K, N>& b, const rt<float, M, N, layout::row>& c) {
+                                       const st<bf16, K, N, PAD>& b, const rt<float, M, N, layout::row>& c) {
     const int i16 = lane() & 15, b16 = lane() >> 4;
     const int srow = 4 * (b16 >> 1) + (i16 >> 2), scol = 16 * (b16 & 1) + 4 * (i16 & 3);
     constexpr int KS = K / 16, NF = (N / 32) * KS, P = kStreamAhead;

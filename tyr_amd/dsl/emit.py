@@ -119,6 +119,30 @@ def infer_rv_layouts(kernel: Kernel) -> Dict[VarId, str]:
 
 _DTYPE_BYTES = {"Float32": 4, "BFloat16": 2, "Float16": 2, "FP8E4M3": 1, "FP8E5M2": 1}
 
+# Padding bytes behind every row of an LDS tile (a multiple of 16: rows stay 16-byte aligned for the 16-byte global <-> LDS
+# moves).  The fragment accesses of this tile library are 8 bytes per lane, 16 lanes to an LDS cycle; which row pitch keeps
+# those apart depends on who the 16 lanes are:
+#   row fragments (lane = row; tiles declared Row): 16 consecutive rows x 2 dwords -- a pitch of 4 dwords mod 64 is conflict-free
+#     on 64 banks, which is what a row of 128 / 256 / 512 bytes gets from 16 bytes of padding;
+#   transposing reads (tiles declared Col, bf16): 4 consecutive rows x four 8-byte column groups -- the rows must land 8 dwords
+#     apart mod 32, i.e. 32 bytes of padding behind rows of 64 / 128 / 256 bytes.
+_PAD_OVERRIDE = {}
+
+
+def st_pad_bytes(d: Stmt) -> int:
+    """Row padding of the LDS tile declared by `d` (a declST statement)."""
+    key = (d.dtype, d.layout)
+    if key in _PAD_OVERRIDE:
+        return _PAD_OVERRIDE[key]
+    if d.layout == "Col" and _DTYPE_BYTES.get(d.dtype) == 2:
+        return 32
+    return 16
+
+
+def st_bytes(d: Stmt) -> int:
+    """Bytes an LDS tile occupies (rounded up to 16)."""
+    return (d.rows * (d.cols * _DTYPE_BYTES[d.dtype] + st_pad_bytes(d)) + 15) // 16 * 16
+
 
 def _st_uses(s: Stmt, tiles) -> set:
     """LDS tiles a (non-compound) statement touches."""
@@ -144,7 +168,7 @@ def lds_plan(kernel: Kernel) -> Dict[VarId, int]:
         b = _DTYPE_BYTES.get(d.dtype)
         if b is None:
             return {}
-        size[v] = (d.rows * (d.cols * b + 16) + 15) // 16 * 16
+        size[v] = st_bytes(d)
     live: Dict[VarId, List[int]] = {}
     pos = [0]
 
@@ -195,7 +219,7 @@ def _lds_regions(kernel: Kernel, plan: Dict[VarId, int]) -> Dict[VarId, Any]:
     if not plan:
         return {}
     decl = {s.v: s for s in walk(kernel.body) if s.op == "declST"}
-    size = {v: (d.rows * (d.cols * _DTYPE_BYTES[d.dtype] + 16) + 15) // 16 * 16 for v, d in decl.items()}
+    size = {v: st_bytes(d) for v, d in decl.items()}
     root = {v: v for v in plan}
 
     def find(v):
@@ -539,7 +563,7 @@ class _Emitter:
         if not self.group:
             return 1
         decl = {t.v: t for t in walk(self.k.body) if t.op == "declST"}
-        size = {v: (d.rows * (d.cols * _DTYPE_BYTES.get(d.dtype, 4) + 16) + 15) // 16 * 16 for v, d in decl.items()}
+        size = {v: st_bytes(d) for v, d in decl.items()}
         lds = max((off + size[v] for v, off in self.lds.items()), default=0) if self.lds else sum(size.values())
         if 2 * lds > 160 * 1024:
             return 1
@@ -574,7 +598,8 @@ class _Emitter:
             #  registers held; where the tile is written first the compiler drops the zeros)
             return f"{ind}rt<{_cpp_type(s.dtype)}, {rows}, {s.cols}, layout::{s.layout.lower()}> {I(s.v)}{{}};\n"
         if op == "declST":
-            ty = f"st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}>"
+            pad = st_pad_bytes(s)
+            ty = f"st<{_cpp_type(s.dtype)}, {s.rows}, {s.cols}" + (f", {pad}>" if pad != 16 else ">")
             if s.v in self.lds:
                 return f"{ind}{ty}& {I(s.v)} = *reinterpret_cast<{ty}*>(tyr_lds_pool + {self.lds[s.v]});\n"
             return f"{ind}__shared__ {ty} {I(s.v)};\n"
@@ -996,8 +1021,7 @@ class _Emitter:
         pool = ""
         if self.lds:
             decl = {t.v: t for t in walk(self.k.body) if t.op == "declST"}
-            total = max(off + (decl[v].rows * (decl[v].cols * _DTYPE_BYTES[decl[v].dtype] + 16) + 15) // 16 * 16
-                        for v, off in self.lds.items())
+            total = max(off + st_bytes(decl[v]) for v, off in self.lds.items())
             pool = (f"  // LDS tiles whose live ranges do not intersect share these bytes\n"
                     f"  __shared__ __attribute__((aligned(16))) unsigned char tyr_lds_pool[{total}];\n")
         head = ""
