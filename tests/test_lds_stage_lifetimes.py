@@ -242,8 +242,8 @@ def test_three_stages_would_not_be_enough_for_the_dkv_kernel():
 # ------------------------------------------------------------------ gemm_bf16_fast_kernel / gemm_fp8_fast_kernel
 def gemm_wave(KT, ksteps):
     """Two stages S0 S1, each an A and a B slice.  Slice kt+1 is requested during the first k-steps of slice kt; the
-    fragments of k-step s+1 are read under the products of k-step s; after the first product row of the last k-step the
-    workgroup waits, synchronises and reads the first fragments of the next slice.  The request and the reads past the
+    fragments of k-step s+1 are read under the products of k-step s; inside the last k-step (bf16: after its second product
+    row, fp8: before its last) the workgroup waits, synchronises and reads the first fragments of the next slice.  The request and the reads past the
     last slice touch the idle stage and are never used (modelled: the request, as it is really issued; not the reads).
     The epilogue stages C through the front of the LDS block (stage 0)."""
     t = Trace()
@@ -268,7 +268,8 @@ def gemm_wave(KT, ksteps):
     return t
 
 
-@pytest.mark.parametrize("ksteps", [4, 2])          # bf16: four k-steps of 16 per 64-wide slice; fp8: two of 64 per 128-byte slice
+# eight waves; bf16: four k-steps of 16 per 64-wide slice; fp8: two k-steps of 64 per 128-byte slice
+@pytest.mark.parametrize("ksteps,waves", [(4, 8), (2, 8)])
 @pytest.mark.parametrize("KT", [1, 2, 3, 4, 63, 64])
-def test_gemm_fast_kernels(KT, ksteps):
-    assert violations([gemm_wave(KT, ksteps) for _ in range(4)]) == []
+def test_gemm_fast_kernels(KT, ksteps, waves):
+    assert violations([gemm_wave(KT, ksteps) for _ in range(waves)]) == []

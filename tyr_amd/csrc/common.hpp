@@ -199,13 +199,16 @@ __device__ __forceinline__ bf16x4 ds_read_tr16(const void* lds_ptr) {
 // LDS scratch (32 rows x 272 B) so that the global stores are 16 bytes per lane along rows.
 constexpr int kEpilogueScratchBytes = 32 * 272;
 // rows / cols = how much of the 128x128 quadrant lies inside C (cols a multiple of 8).
-__device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], float scale, unsigned char* scratch,
+// NJ = 32-column tiles of the wave's block (4: a 128x128 quadrant; 2: 128x64).
+template <int NJ>
+__device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][NJ], float scale, unsigned char* scratch,
                                                     uint16_t* c_quadrant, int ldc, int lane, int rows, int cols) {
     const int r = lane & 31, g = lane >> 5;
+    constexpr int CH = NJ * 4;                           // 16-byte chunks per row of the block
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 u32x2 v;
@@ -214,11 +217,11 @@ __device__ __forceinline__ void store_quadrant_bf16(const f32x16 (&acc)[4][4], f
                 *reinterpret_cast<u32x2*>(scratch + r * 272 + (j * 32 + q4 * 8 + g * 4) * 2) = v;
             }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const int row = (lane >> 4) + 4 * k;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * 272 + (lane & 15) * 16);
-            if (i * 32 + row < rows && (lane & 15) * 8 < cols)
-                st_global_16(c_quadrant + (size_t)(i * 32 + row) * ldc + (lane & 15) * 8, v);
+        for (int k = 0; k < 32 * CH / 64; ++k) {
+            const int row = lane / CH + (64 / CH) * k;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + row * 272 + (lane % CH) * 16);
+            if (i * 32 + row < rows && (lane % CH) * 8 < cols)
+                st_global_16(c_quadrant + (size_t)(i * 32 + row) * ldc + (lane % CH) * 8, v);
         }
     }
 }
@@ -235,7 +238,8 @@ struct GemmEpilogue {
 // One wave's 128x128 accumulator quadrant (layout as in store_quadrant_bf16) written straight from registers:
 // a lane stores the 4 consecutive n of a register group of its row.  gm0 / gn0 = global row / column of the
 // quadrant's first element; M, N = extents of C (row pitch N elements).
-__device__ __forceinline__ void store_quadrant_ex(const f32x16 (&acc)[4][4], const GemmEpilogue& ep, void* C, int M, int N,
+template <int NJ>
+__device__ __forceinline__ void store_quadrant_ex(const f32x16 (&acc)[4][NJ], const GemmEpilogue& ep, void* C, int M, int N,
                                                   int gm0, int gn0, int lane) {
     const int r = lane & 31, g = lane >> 5;
 #pragma unroll
@@ -244,7 +248,7 @@ __device__ __forceinline__ void store_quadrant_ex(const f32x16 (&acc)[4][4], con
         if (gm >= M) continue;
         const float rs = ep.scale * (ep.row_scale ? ep.row_scale[gm] : 1.0f);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int gn = gn0 + j * 32 + q4 * 8 + g * 4;

@@ -193,7 +193,7 @@ __global__ __launch_bounds__(gemm::THREADS) void gemm_bf16_kernel(
 // one n) are gathered by the transposing LDS read.  Fragments for k-step s+1 are requested before
 // the 16 MFMAs of k-step s are issued.
 namespace gemm2 {
-constexpr int BM = 256, BN = 256, BK = 64, THREADS = 256;
+constexpr int BM = 256, BN = 256, BK = 64, THREADS = 512;
 constexpr int A_TILE = BM * BK * 2;                  // 32 KiB: [256 m][8 chunks]
 constexpr int B_TILE = BN * BK * 2;                  // 32 KiB: [64 k][32 chunks] or [256 n][8 chunks]
 constexpr int STAGE = A_TILE + B_TILE;
@@ -202,7 +202,7 @@ constexpr int GROUP_M = 4;
 }  // namespace gemm2
 
 template <bool TRANS_B, bool K_TAIL>
-__global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
+__global__ __launch_bounds__(gemm2::THREADS, 1) void gemm_bf16_fast_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, int tiles_m, int tiles_n, long stride_a, long stride_b, long stride_c) {
     using namespace gemm2;
@@ -212,9 +212,9 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     C += (size_t)blockIdx.y * stride_c;
 
     const int t = threadIdx.x;
-    const int lane = t & 63, w = t >> 6;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r = lane & 31, g = lane >> 5;
-    const int wm = w >> 1, wn = w & 1;
+    const int wm = w >> 2, wn = w & 3;                 // eight waves: wave (wm, wn) owns 128 rows x 64 columns
 
     const uint32_t nblk = (uint32_t)tiles_m * (uint32_t)tiles_n;
     const uint32_t pid = xcd_remap(blockIdx.x, nblk);
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     const int tn = (int)((pid % per_group) / gsz);
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // ---- global -> LDS requests.  Each wave owns a quarter of each tile: 8 instructions of 1 KiB.
+    // ---- global -> LDS requests.  Each wave owns an eighth of each tile: 4 instructions of 1 KiB.
     // A (and B when TRANS_B): 8 rows of 128 B per instruction; chunk c of row m is stored at
     // position c ^ ((m >> 1) & 7), so 16 consecutive rows put one logical chunk on all 64 banks.  B when !TRANS_B: 2 rows of 512 B per instruction; chunk c of row k is
     // stored at position c ^ ((k & 3) << 2).
@@ -238,39 +238,39 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
         //  off the per-lane offsets below, and those must not go negative)
         : make_raw_rsrc(B + n0 - 1536, (uint32_t)min(((size_t)K * N - n0) * 2 + 3072, (size_t)0xffffffffu));
-    int a_voff[8], b_voff[8];
+    int a_voff[4], b_voff[4];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-        const int row = (w * 8 + m) * 8 + (lane >> 3);
+    for (int m = 0; m < 4; ++m) {
+        const int row = (w * 4 + m) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);
-        // (1024 (m % 4) is taken off: the request carries it as its immediate offset, see issue_half)
-        a_voff[m] = row * K * 2 + c * 16 - 1024 * (m & 3);
+        // (1024 m is taken off: the request carries it as its immediate offset, see issue)
+        a_voff[m] = row * K * 2 + c * 16 - 1024 * m;
         if (TRANS_B) {
-            b_voff[m] = row * K * 2 + c * 16 - 1024 * (m & 3);
+            b_voff[m] = row * K * 2 + c * 16 - 1024 * m;
         } else {
-            const int krow = (w * 8 + m) * 2 + (lane >> 5);
+            const int krow = (w * 4 + m) * 2 + (lane >> 5);
             const int cb = (lane & 31) ^ ((krow & 3) << 2);
-            b_voff[m] = krow * N * 2 + cb * 16 - 1024 * (m & 3) + 3072;
+            b_voff[m] = krow * N * 2 + cb * 16 - 1024 * m + 3072;
         }
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
-    // half h (0..1) of the requests for slice kt into stage st: 4 A + 4 B instructions, each group of
-    // four behind one M0 write (the immediate offset steps the LDS destination by a kilobyte)
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 4096u);
+    // the wave's requests for slice kt into stage st: part 0 the A tile, part 1 the B tile, four instructions
+    // behind one M0 write each (the immediate offset steps the LDS destination by a kilobyte)
     const int KT = (K + BK - 1) / BK;
-    auto issue_half = [&](int st, int kt, int h, int part = 2) {
+    auto issue = [&](int st, int kt, int part) {
         const int a_soff = kt * BK * 2;
         const int b_soff = TRANS_B ? kt * BK * 2 : kt * BK * N * 2;
-        const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
-        int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
-        int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
+        int av[4] = {a_voff[0], a_voff[1], a_voff[2], a_voff[3]};
+        int bv[4] = {b_voff[0], b_voff[1], b_voff[2], b_voff[3]};
         if (K_TAIL && kt == KT - 1) {
             // ragged last slice (K % 8 == 0): the 16-byte chunks of a row at k >= K belong to the next
             // row and must read as zeros; rows k >= K of a [K,N] B are past its descriptor already
             const int chunks = (K - kt * BK) >> 3;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int row = (w * 8 + 4 * h + i) * 8 + (lane >> 3);
+                const int row = (w * 4 + i) * 8 + (lane >> 3);
                 const int c = (lane & 7) ^ ((row >> 1) & 7);
                 if (c >= chunks) {
                     av[i] = (int)0x80000000u;
@@ -278,8 +278,8 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
                 }
             }
         }
-        if (part != 1) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
-        if (part != 0) load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
+        if (part == 0) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        else           load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses
@@ -289,58 +289,63 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
     for (int s = 0; s < 4; ++s) a_roff[s] = (wm * 128 + r) * 128 + (((2 * s + g) ^ ((r >> 1) & 7)) * 16);
     // B fragment, TRANS_B: like A with n rows.  Otherwise (row-major [k][n]) via the transposing
     // read: as a source lane this lane points at k row 8(b/2) + 4h + j (j = (lane%16)/4) of the
-    // k-step, 8 bytes at n = wn*128 + 32jt + 16(b&1) + 4(lane%4); jt enters through the swizzle.
+    // k-step, 8 bytes at n = wn*64 + 32jt + 16(b&1) + 4(lane%4); jt enters through the swizzle.
     int b_roff[4];
     if (TRANS_B) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) b_roff[s] = A_TILE + (wn * 128 + r) * 128 + (((2 * s + g) ^ ((r >> 1) & 7)) * 16);
+        for (int s = 0; s < 4; ++s) b_roff[s] = A_TILE + (wn * 64 + r) * 128 + (((2 * s + g) ^ ((r >> 1) & 7)) * 16);
     } else {
         const int i16 = lane & 15, b16 = lane >> 4;
         const int js = i16 >> 2, qs = i16 & 3;
         const int krow = 8 * (b16 >> 1) + js;
 #pragma unroll
-        for (int jt = 0; jt < 4; ++jt) {
-            const int c = wn * 16 + 4 * jt + 2 * (b16 & 1) + (qs >> 1);
+        for (int jt = 0; jt < 2; ++jt) {
+            const int c = wn * 8 + 4 * jt + 2 * (b16 & 1) + (qs >> 1);
             b_roff[jt] = A_TILE + krow * 512 + ((c ^ (js << 2)) * 16) + (qs & 1) * 8;
         }
+        b_roff[2] = b_roff[3] = 0;
     }
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // fragment pair i of k-step s: the A fragment of m tile i and the B fragment of n tile i
-    auto read_pair = [&](const unsigned char* St, int s, int i, bf16x8& fa, bf16x8& fb) {
+    // fragments of k-step s: A of m tile i, B of n tile j
+    auto read_a = [&](const unsigned char* St, int s, int i, bf16x8& fa) {
         fa = *reinterpret_cast<const bf16x8*>(St + a_roff[s] + i * 32 * 128);
+    };
+    auto read_b = [&](const unsigned char* St, int s, int j, bf16x8& fb) {
         if (TRANS_B) {
-            fb = *reinterpret_cast<const bf16x8*>(St + b_roff[s] + i * 32 * 128);
+            fb = *reinterpret_cast<const bf16x8*>(St + b_roff[s] + j * 32 * 128);
         } else {
-            const unsigned char* p = St + b_roff[i] + s * 16 * 512;
+            const unsigned char* p = St + b_roff[j] + s * 16 * 512;
             const bf16x4 lo = ds_read_tr16(p);
             const bf16x4 hi = ds_read_tr16(p + 4 * 512);
             fb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
     };
 
-#pragma unroll
-    for (int h = 0; h < 2; ++h) issue_half(0, 0, h);
+    issue(0, 0, 0);
+    issue(0, 0, 1);
     wait_vmcnt0();
     __syncthreads();
 
     // Steady state per slice: the next slice is requested during k-steps 0 and 1; the fragments of
-    // k-step s+1 are read during the MFMAs of k-step s; after the first MFMA row of the last k-step
-    // the workgroup synchronises and reads the first fragments of the next slice.  A wave is alone
-    // on its SIMD, so whatever it issues between two MFMAs is time the matrix pipe may idle: the
-    // requests and the fragment reads are dealt out between the MFMA rows (4 MFMAs, 128 cycles each)
-    // instead of standing in one block before them, and the scheduling barriers keep that order.
+    // k-step s+1 are read during the MFMAs of k-step s; in the middle of the last k-step the workgroup
+    // waits for the requests, synchronises and reads the first fragments of the next slice.  Two waves
+    // share a SIMD, so what one waits for is covered by the other's MFMAs; requests and fragment reads
+    // are still dealt out between the MFMA rows (2 MFMAs, 64 cycles each) and the scheduling barriers
+    // keep that order.
     // (Past the last slice the requests and reads touch the idle stage / stale data and are never used.)
-    bf16x8 af[2][4], bf[2][4];
+    bf16x8 af[2][4], bf[2][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) read_pair(lds, 0, i, af[0][i], bf[0][i]);
+    for (int i = 0; i < 4; ++i) read_a(lds, 0, i, af[0][i]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) read_b(lds, 0, j, bf[0][j]);
 #define TYR_FENCE __builtin_amdgcn_sched_barrier(0)
     for (int kt = 0; kt < KT; ++kt) {
         const int st = kt & 1;
@@ -348,7 +353,7 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
         const unsigned char* Sn = lds + (st ^ 1) * STAGE;
         auto row = [&](int b, int i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[b][j], af[b][i], acc[i][j]);
+            for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16_bf16(bf[b][j], af[b][i], acc[i][j]);
         };
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
@@ -356,30 +361,33 @@ __global__ __launch_bounds__(gemm2::THREADS) void gemm_bf16_fast_kernel(
             if (s < 3) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (s < 2 && i < 2) issue_half(st ^ 1, kt + 1, s, i);
-                    read_pair(St, s + 1, i, af[nb][i], bf[nb][i]);
+                    if (s < 2 && i == 0) issue(st ^ 1, kt + 1, s);
+                    read_a(St, s + 1, i, af[nb][i]);
+                    if (i < 2) read_b(St, s + 1, i, bf[nb][i]);
                     TYR_FENCE; row(cb, i); TYR_FENCE;
                 }
             } else {
                 row(cb, 0); TYR_FENCE;
+                row(cb, 1); TYR_FENCE;
                 wait_vmcnt0();
                 __syncthreads();
-                read_pair(Sn, 0, 0, af[nb][0], bf[nb][0]);
-                read_pair(Sn, 0, 1, af[nb][1], bf[nb][1]);
-                TYR_FENCE; row(cb, 1); TYR_FENCE;
-                read_pair(Sn, 0, 2, af[nb][2], bf[nb][2]);
-                read_pair(Sn, 0, 3, af[nb][3], bf[nb][3]);
+                read_a(Sn, 0, 0, af[nb][0]);
+                read_b(Sn, 0, 0, bf[nb][0]);
+                read_b(Sn, 0, 1, bf[nb][1]);
                 TYR_FENCE; row(cb, 2); TYR_FENCE;
-                row(cb, 3); TYR_FENCE;
+                read_a(Sn, 0, 1, af[nb][1]);
+                read_a(Sn, 0, 2, af[nb][2]);
+                read_a(Sn, 0, 3, af[nb][3]);
+                TYR_FENCE; row(cb, 3); TYR_FENCE;
             }
         }
     }
 #undef TYR_FENCE
 
     // ---- epilogue (all requests have landed and every wave is past its last fragment read)
-    store_quadrant_bf16(acc, 1.0f, lds + w * kEpilogueScratchBytes,
-                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
-                        M - (m0 + wm * 128), N - (n0 + wn * 128));
+    store_quadrant_bf16<2>(acc, 1.0f, lds + w * kEpilogueScratchBytes,
+                           C + (size_t)(m0 + wm * 128) * N + n0 + wn * 64, N, lane,
+                           M - (m0 + wm * 128), N - (n0 + wn * 64));
 }
 
 int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K, int trans_b,
@@ -407,7 +415,7 @@ int launch_gemm_bf16(const void* a, const void* b, void* c, int M, int N, int K,
                 reinterpret_cast<const void*>(&gemm_bf16_fast_kernel<TB, KT>),                    \
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm2::LDS_BYTES);                    \
             if (attr != hipSuccess) return -1;                                                    \
-            hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB, KT>), grid, block, gemm2::LDS_BYTES, stream, \
+            hipLaunchKernelGGL((gemm_bf16_fast_kernel<TB, KT>), grid, dim3(gemm2::THREADS), gemm2::LDS_BYTES, stream, \
                                A, Bp, Cp, M, N, K, tiles_m, tiles_n, (long)stride_a, (long)stride_b,  \
                                (long)stride_c);                                                   \
         } while (0)

@@ -7,10 +7,12 @@
 // (e4m3 x e4m3 -> f32 -> bf16) and Tyr/GPU/Kernels/GemmCommon.lean:135-144 (one scalar
 // multiplied into the f32 accumulator tile before the store).
 //
-// Same skeleton as the bf16 GEMM: 256x256 output tile per 4-wave workgroup, K in slices of
-// 128 bytes, k-contiguous padded LDS rows for both operands, two LDS stages with register
-// prefetch, one barrier per slice.  For B stored [K,N] the loader transposes 16(k) x 8(n) byte
-// blocks in registers (two levels of v_perm_b32) on the way to LDS.
+// Two kernels.  The general one has the skeleton of the bf16 GEMM's general kernel: 256x256 output tile per
+// 4-wave workgroup, K in slices of 128 bytes, k-contiguous padded LDS rows for both operands, two LDS
+// stages with register prefetch, one barrier per slice; for B stored [K,N] its loader transposes
+// 16(k) x 8(n) byte blocks in registers (two levels of v_perm_b32) on the way to LDS.  The fast one
+// (further down; every shape whose offsets fit 32 bits takes it) moves slices straight into LDS and runs
+// the same tile with eight waves.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -206,8 +208,10 @@ __global__ __launch_bounds__(gemm8::THREADS) void gemm_fp8_kernel(
 // Fast path for K % 16 == 0 (any M; N % 16 == 0; a last slice shorter than 128 is zero-filled): slices go from global memory straight
 // into LDS, unpadded rows with XOR-swizzled 16-byte chunks; a [K,N] B stays row-major in LDS and
 // its fragments (32 consecutive k for one n) are gathered with the byte-transposing LDS read.
+// Eight waves, two per SIMD: wave (wm, wn) owns 128 rows x 64 columns of the tile (4 x 2 MFMA tiles, 128 accumulator
+// registers), so that what one wave waits for (LDS fragments, the slice barrier) is covered by the other's MFMAs.
 namespace gemm8f {
-constexpr int BM = 256, BN = 256, BK = 128, THREADS = 256;
+constexpr int BM = 256, BN = 256, BK = 128, THREADS = 512;
 constexpr int A_TILE = BM * BK;                      // 32 KiB: [256 m][8 chunks]
 constexpr int B_TILE = BN * BK;                      // 32 KiB: [128 k][16 chunks] or [256 n][8 chunks]
 constexpr int STAGE = A_TILE + B_TILE;
@@ -216,7 +220,7 @@ constexpr int GROUP_M = 4;
 }  // namespace gemm8f
 
 template <bool TRANS_B, bool K_TAIL>
-__global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
+__global__ __launch_bounds__(gemm8f::THREADS, 1) void gemm_fp8_fast_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, int tiles_m, int tiles_n, GemmEpilogue ep) {
     const float scale = ep.scale;
@@ -224,9 +228,9 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int t = threadIdx.x;
-    const int lane = t & 63, w = t >> 6;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r = lane & 31, g = lane >> 5;
-    const int wm = w >> 1, wn = w & 1;
+    const int wm = w >> 2, wn = w & 3;
 
     const uint32_t nblk = (uint32_t)tiles_m * (uint32_t)tiles_n;
     const uint32_t pid = xcd_remap(blockIdx.x, nblk);
@@ -238,49 +242,47 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
     const int tn = (int)((pid % per_group) / gsz);
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // ---- global -> LDS requests (8 instructions of 1 KiB per wave and tile).
+    // ---- global -> LDS requests (4 instructions of 1 KiB per wave and operand tile).
     // A (and B when TRANS_B): 8 rows of 128 B per instruction, chunk c of row m at c ^ ((m>>1)&7).
     // B when !TRANS_B: 4 rows of 256 B per instruction, chunk c of row k at c ^ ((k&7)<<1).
     // (a descriptor spans the tile's rows only and stays below 2 GiB, so that the offset 2^31 given to
-    //  the chunks past K of a ragged last slice is out of range whatever is added to it)
+    //  the chunks past K of a ragged last slice is out of range whatever is added to it; the [K,N] B
+    //  descriptor is shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
+    //  off the per-lane offsets below, and those must not go negative)
     const u32x4 a_rsrc = make_raw_rsrc(A + (size_t)m0 * K, (uint32_t)((size_t)min(M - m0, BM) * K));
     const u32x4 b_rsrc = TRANS_B
         ? make_raw_rsrc(B + (size_t)n0 * K, (uint32_t)((size_t)min(N - n0, BN) * K))
-        // (descriptor shifted down by 3072 bytes: with few columns a row is shorter than the kilobytes taken
-        //  off the per-lane offsets below, and those must not go negative)
         : make_raw_rsrc(B + n0 - 3072, (uint32_t)min((size_t)K * N - n0 + 3072, (size_t)0xffffffffu));
-    int a_voff[8], b_voff[8];
+    int a_voff[4], b_voff[4];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-        const int row = (w * 8 + m) * 8 + (lane >> 3);
+    for (int m = 0; m < 4; ++m) {
+        const int row = (w * 4 + m) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);
-        // (1024 (m % 4) is taken off: the request carries it as its immediate offset, see issue_half)
-        a_voff[m] = row * K + c * 16 - 1024 * (m & 3);
+        a_voff[m] = row * K + c * 16 - 1024 * m;
         if (TRANS_B) {
-            b_voff[m] = row * K + c * 16 - 1024 * (m & 3);
+            b_voff[m] = row * K + c * 16 - 1024 * m;
         } else {
-            const int krow = (w * 8 + m) * 4 + (lane >> 4);
+            const int krow = (w * 4 + m) * 4 + (lane >> 4);
             const int cb = (lane & 15) ^ ((krow & 7) << 1);
-            b_voff[m] = krow * N + cb * 16 - 1024 * (m & 3) + 3072;
+            b_voff[m] = krow * N + cb * 16 - 1024 * m + 3072;
         }
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 8192u);
+    const uint32_t wave_dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)w * 4096u);
     const int KT = (K + BK - 1) / BK;
-    auto issue_half = [&](int st, int kt, int h, int part = 2) {
+    auto issue = [&](int st, int kt, int part) {         // part 0: the A tile, 1: the B tile
         const int a_soff = kt * BK;
         const int b_soff = TRANS_B ? kt * BK : kt * BK * N;
-        // four requests behind one M0 write: the immediate offset steps the LDS destination by a kilobyte
-        const uint32_t dst = wave_dst + (uint32_t)st * STAGE + (uint32_t)h * 4096u;
-        int av[4] = {a_voff[4 * h], a_voff[4 * h + 1], a_voff[4 * h + 2], a_voff[4 * h + 3]};
-        int bv[4] = {b_voff[4 * h], b_voff[4 * h + 1], b_voff[4 * h + 2], b_voff[4 * h + 3]};
+        const uint32_t dst = wave_dst + (uint32_t)st * STAGE;
+        int av[4] = {a_voff[0], a_voff[1], a_voff[2], a_voff[3]};
+        int bv[4] = {b_voff[0], b_voff[1], b_voff[2], b_voff[3]};
         if (K_TAIL && kt == KT - 1) {
             // ragged last slice (K % 16 == 0): the 16-byte chunks of a row at k >= K belong to the next
             // row and must read as zeros; rows k >= K of a [K,N] B are past its descriptor already
             const int chunks = (K - kt * BK) >> 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int row = (w * 8 + 4 * h + i) * 8 + (lane >> 3);
+                const int row = (w * 4 + i) * 8 + (lane >> 3);
                 const int c = (lane & 7) ^ ((row >> 1) & 7);
                 if (c >= chunks) {
                     av[i] = (int)0x80000000u;
@@ -288,8 +290,8 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
                 }
             }
         }
-        if (part != 1) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
-        if (part != 0) load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
+        if (part == 0) load_global_to_lds_16xN<4>(a_rsrc, dst, av, a_soff);
+        else           load_global_to_lds_16xN<4>(b_rsrc, dst + A_TILE, bv, b_soff);
     };
 
     // ---- fragment addresses.  k-step s covers bytes [64s, 64s+64) of a row; lane group g takes
@@ -300,59 +302,60 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
 #pragma unroll
         for (int h = 0; h < 2; ++h)
             a_roff[s][h] = (wm * 128 + r) * 128 + (((4 * s + 2 * g + h) ^ ((r >> 1) & 7)) * 16);
-    int b_roff[4];    // TRANS_B: [s][h] like A.  Otherwise [jt]: source-lane address for n tile jt.
+    int b_roff[4];    // TRANS_B: [s][h] like A.  Otherwise [jt] (two used): source-lane address for n tile jt.
     if (TRANS_B) {
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                b_roff[2 * s + h] = A_TILE + (wn * 128 + r) * 128 + (((4 * s + 2 * g + h) ^ ((r >> 1) & 7)) * 16);
+                b_roff[2 * s + h] = A_TILE + (wn * 64 + r) * 128 + (((4 * s + 2 * g + h) ^ ((r >> 1) & 7)) * 16);
     } else {
         // As a source lane of the byte-transposing read: k row 32(b/2) + (lane%16)/2 (+64s + 8h),
-        // 8 bytes at n = wn*128 + 32jt + 16(b&1) + 8(lane%2).
+        // 8 bytes at n = wn*64 + 32jt + 16(b&1) + 8(lane%2).
         const int i16 = lane & 15, b16 = lane >> 4;
         const int js = i16 >> 1, qs = i16 & 1;
         const int krow = 32 * (b16 >> 1) + js;
 #pragma unroll
-        for (int jt = 0; jt < 4; ++jt) {
-            const int c = wn * 8 + 2 * jt + (b16 & 1);
+        for (int jt = 0; jt < 2; ++jt) {
+            const int c = wn * 4 + 2 * jt + (b16 & 1);
             b_roff[jt] = A_TILE + krow * 256 + ((c ^ (js << 1)) * 16) + qs * 8;
         }
+        b_roff[2] = b_roff[3] = 0;
     }
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    issue_half(0, 0, 0);
-    issue_half(0, 0, 1);
+    issue(0, 0, 0);
+    issue(0, 0, 1);
     wait_vmcnt0();
     __syncthreads();
 
-    // Per slice: k-step 0 requests the next slice and reads the fragments of k-step 1; after the
-    // first MFMA row of k-step 1 the workgroup synchronises and reads the first fragments of the
-    // next slice.  A wave is alone on its SIMD, so whatever it issues between two MFMAs is time the
-    // matrix pipe may idle: the requests and the fragment reads are therefore dealt out between the
-    // MFMA rows (4 MFMAs, 256 cycles each) instead of standing in one block before them, and the
-    // scheduling barriers keep that order.
-    i32x8 af[2][4], bf[2][4];
-    // fragment pair i of k-step s: the A fragment of m tile i and the B fragment of n tile i
-    auto read_pair = [&](const unsigned char* St, int s, int i, i32x8& a, i32x8& b) {
-        {
-            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + a_roff[s][0] + i * 32 * 128);
-            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + a_roff[s][1] + i * 32 * 128);
-            a = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-        }
+    // Per slice: k-step 0 requests the next slice and reads the fragments of k-step 1; before the last MFMA row of
+    // k-step 1 the workgroup waits for the requests, synchronises and reads the first fragments of the next slice.
+    // The wait stands as late as the fragment reads behind it allow: the slice requests then have almost a whole slice
+    // to land (after the first MFMA row of k-step 1, where it stood first, 8192^3 took 6 % longer: a fifth of the
+    // requests miss the L2 and arrive later than that).  Requests and fragment reads are dealt out between the MFMA
+    // rows (2 MFMAs, 128 cycles each) and the scheduling barriers keep that order.
+    // (Past the last slice the requests and reads touch the idle stage / stale data and are never used.)
+    i32x8 af[2][4], bf[2][2];
+    auto read_a = [&](const unsigned char* St, int s, int i, i32x8& a) {
+        const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + a_roff[s][0] + i * 32 * 128);
+        const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + a_roff[s][1] + i * 32 * 128);
+        a = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+    };
+    auto read_b = [&](const unsigned char* St, int s, int j, i32x8& b) {
         if (TRANS_B) {
-            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s] + i * 32 * 128);
-            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s + 1] + i * 32 * 128);
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s] + j * 32 * 128);
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(St + b_roff[2 * s + 1] + j * 32 * 128);
             b = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
         } else {
-            const unsigned char* p = St + b_roff[i] + s * 64 * 256;
+            const unsigned char* p = St + b_roff[j] + s * 64 * 256;
             const u32x2 y0 = ds_read_tr8(p);
             const u32x2 y1 = ds_read_tr8(p + 8 * 256);
             const u32x2 y2 = ds_read_tr8(p + 16 * 256);
@@ -361,7 +364,9 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
         }
     };
 #pragma unroll
-    for (int i = 0; i < 4; ++i) read_pair(lds, 0, i, af[0][i], bf[0][i]);
+    for (int i = 0; i < 4; ++i) read_a(lds, 0, i, af[0][i]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) read_b(lds, 0, j, bf[0][j]);
 #define TYR_FENCE __builtin_amdgcn_sched_barrier(0)
     for (int kt = 0; kt < KT; ++kt) {
         const int st = kt & 1;
@@ -369,38 +374,39 @@ __global__ __launch_bounds__(gemm8f::THREADS) void gemm_fp8_fast_kernel(
         const unsigned char* Sn = lds + (st ^ 1) * STAGE;
         auto row = [&](int s, int i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
+            for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x64_e4m3(bf[s][j], af[s][i], acc[i][j]);
         };
         // The first MFMA row goes out before any fragment of the next k-step is requested: at the top of the loop
         // the compiler waits for every LDS read in flight (it cannot count across the back edge), and with fresh
         // requests in front of that wait the wave would sit out their latency once per slice.
-        issue_half(st ^ 1, kt + 1, 0, 0);
+        issue(st ^ 1, kt + 1, 0);
         TYR_FENCE; row(0, 0); TYR_FENCE;
-        read_pair(St, 1, 0, af[1][0], bf[1][0]);
-        issue_half(st ^ 1, kt + 1, 0, 1);
-        read_pair(St, 1, 1, af[1][1], bf[1][1]); TYR_FENCE; row(0, 1); TYR_FENCE;
-        issue_half(st ^ 1, kt + 1, 1, 0);
-        read_pair(St, 1, 2, af[1][2], bf[1][2]); TYR_FENCE; row(0, 2); TYR_FENCE;
-        issue_half(st ^ 1, kt + 1, 1, 1);
-        read_pair(St, 1, 3, af[1][3], bf[1][3]); TYR_FENCE; row(0, 3); TYR_FENCE;
+        read_a(St, 1, 0, af[1][0]); read_b(St, 1, 0, bf[1][0]);
+        issue(st ^ 1, kt + 1, 1);
+        read_b(St, 1, 1, bf[1][1]); TYR_FENCE; row(0, 1); TYR_FENCE;
+        read_a(St, 1, 1, af[1][1]); TYR_FENCE; row(0, 2); TYR_FENCE;
+        read_a(St, 1, 2, af[1][2]);
+        read_a(St, 1, 3, af[1][3]); TYR_FENCE; row(0, 3); TYR_FENCE;
         row(1, 0); TYR_FENCE;
+        row(1, 1); TYR_FENCE;
+        row(1, 2); TYR_FENCE;
         wait_vmcnt0();
         __syncthreads();
-        read_pair(Sn, 0, 0, af[0][0], bf[0][0]);
-        read_pair(Sn, 0, 1, af[0][1], bf[0][1]); TYR_FENCE; row(1, 1); TYR_FENCE;
-        read_pair(Sn, 0, 2, af[0][2], bf[0][2]);
-        read_pair(Sn, 0, 3, af[0][3], bf[0][3]); TYR_FENCE; row(1, 2); TYR_FENCE;
-        row(1, 3); TYR_FENCE;
+        read_a(Sn, 0, 0, af[0][0]); read_b(Sn, 0, 0, bf[0][0]);
+        read_b(Sn, 0, 1, bf[0][1]);
+        read_a(Sn, 0, 1, af[0][1]);
+        read_a(Sn, 0, 2, af[0][2]);
+        read_a(Sn, 0, 3, af[0][3]); TYR_FENCE; row(1, 3); TYR_FENCE;
     }
 #undef TYR_FENCE
 
     if (!ep.plain_bf16()) {
-        store_quadrant_ex(acc, ep, C, M, N, m0 + wm * 128, n0 + wn * 128, lane);
+        store_quadrant_ex<2>(acc, ep, C, M, N, m0 + wm * 128, n0 + wn * 64, lane);
         return;
     }
-    store_quadrant_bf16(acc, scale, lds + w * kEpilogueScratchBytes,
-                        C + (size_t)(m0 + wm * 128) * N + n0 + wn * 128, N, lane,
-                        M - (m0 + wm * 128), N - (n0 + wn * 128));
+    store_quadrant_bf16<2>(acc, scale, lds + w * kEpilogueScratchBytes,
+                           C + (size_t)(m0 + wm * 128) * N + n0 + wn * 64, N, lane,
+                           M - (m0 + wm * 128), N - (n0 + wn * 64));
 }
 
 int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K, float scale,
@@ -428,7 +434,7 @@ int launch_gemm_fp8(const void* aq, const void* bq, void* c, int M, int N, int K
                 reinterpret_cast<const void*>(&gemm_fp8_fast_kernel<TB, KT>),                     \
                 hipFuncAttributeMaxDynamicSharedMemorySize, gemm8f::LDS_BYTES);                   \
             if (attr != hipSuccess) return -1;                                                    \
-            hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB, KT>), grid, block, gemm8f::LDS_BYTES, stream, \
+            hipLaunchKernelGGL((gemm_fp8_fast_kernel<TB, KT>), grid, dim3(gemm8f::THREADS), gemm8f::LDS_BYTES, stream, \
                                A, Bp, Cp, M, N, K, tiles_m, tiles_n, ep);                         \
         } while (0)
         const bool k_tail = K % gemm8f::BK != 0;
