@@ -140,13 +140,18 @@ def test_conflicting_vector_use_is_an_error():
 def test_nvidia_only_statements_are_refused_and_mma_bookkeeping_is_a_no_op():
     k = dsl.KernelBuilder("tma")
     a = k.allocST("BFloat16", 64, 64)
-    k.emit(stmt("prefetch", a.id))
-    with pytest.raises(dsl.UnsupportedStatement, match="prefetch"):
+    k.emit(stmt("tmaExpect", a.id, 4096))
+    with pytest.raises(dsl.UnsupportedStatement, match="tmaExpect"):
         dsl.emit_kernel(k.build())
     k = dsl.KernelBuilder("fence")
     k.emit(stmt("mmaCommitGroup"))
     k.emit(stmt("mmaAsyncWait", 0))
     assert dsl.emit_kernel(k.build()).count("nothing to do") == 2
+    # the TMA prefetch hint changes no value: it is dropped, not refused
+    k = dsl.KernelBuilder("hint")
+    a = k.allocST("BFloat16", 64, 64)
+    k.emit(stmt("prefetch", a.id))
+    assert "a hint, nothing to do" in dsl.emit_kernel(k.build())
 
 
 def test_launcher_text():

@@ -9,7 +9,8 @@ signature and error strings.
 
 Statements that only exist for NVIDIA hardware paths (TMA, multimem, tcgen05, semaphores, named
 barriers, warp-group election) raise `UnsupportedStatement`; the asynchronous-MMA bookkeeping
-statements are no-ops because an MFMA is complete when its result is read.
+statements are no-ops because an MFMA is complete when its result is read, and the prefetch hint is
+a no-op because it changes no value.
 """
 from __future__ import annotations
 
@@ -37,8 +38,8 @@ REDUCE = {"Max": "op_max", "Min": "op_min", "Sum": "op_add", "Prod": "op_mul"}
 MASK = {"MakeCausal": "keep_causal", "MakeCausalT": "keep_causal_t", "Tril": "keep_tril", "Triu": "keep_triu",
         "RightFill": "keep_right_fill", "LeftFill": "keep_left_fill", "UpperFill": "keep_upper_fill",
         "LowerFill": "keep_lower_fill"}
-NO_OPS = {"mmaFence", "mmaCommitGroup", "mmaAsyncWait", "fenceViewAsyncShared", "fenceProxyAsync"}
-NVIDIA_ONLY = {"declSemaphore", "loadAsync", "storeAsync", "storeAdd", "storeAddAsync", "storeMinAsync", "prefetch",
+NO_OPS = {"mmaFence", "mmaCommitGroup", "mmaAsyncWait", "fenceViewAsyncShared", "fenceProxyAsync", "prefetch"}
+NVIDIA_ONLY = {"declSemaphore", "loadAsync", "storeAsync", "storeAdd", "storeAddAsync", "storeMinAsync",
                "tmaExpect", "tmaLoad", "tmaStore", "loadGlobalAsync", "storeGlobalAsync",
                "multimemLoadReduce", "multimemStore", "multimemRed",
                "tcgen05Mma", "cpAsyncLoad", "tmaLoadAsync", "arrive", "arriveAndWait", "namedBarrierSync",
@@ -588,6 +589,10 @@ class _Emitter:
         op, I = s.op, (lambda v: v.ident)
         if op in NVIDIA_ONLY:
             raise UnsupportedStatement(f"{op} has no gfx950 lowering")
+        if op == "prefetch":
+            # a hint with no effect on values (the reference prints warp::tma::prefetch, EmitNew.lean:239); the tile is
+            # fetched by the load that uses it
+            return f"{ind}// prefetch of {I(s.src)}: a hint, nothing to do\n"
         if op in NO_OPS:
             return f"{ind}// {op}: nothing to do, an MFMA result is complete when it is read\n"
         if op == "declRT":
